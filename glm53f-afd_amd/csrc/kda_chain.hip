@@ -1,0 +1,487 @@
+// KDA recurrent path on gfx950: the decode / verify chain, the replays, the conv-window shift and the
+// checkpoint selection. One workgroup of 256 lanes (4 waves) per (head, request). The per-row arithmetic
+// follows the reference's CPU model operation for operation (crates/glm53f-kda/src/cpu.rs:410-471); what is
+// new is the mapping: every lane streams 128-bit pieces of the state (a value row per 16 or 32 lanes),
+// keeps 64 state values in registers across the rows of a window, and sums over keys inside its wave.
+//
+// Compiled with floating-point contraction off: the state update must not fuse a multiply and an add, so
+// that chain, replay and verify give the same bits (and those of the CPU model).
+
+#include "kda_common.h"
+
+namespace kda {
+namespace {
+
+constexpr int THREADS = 256;
+
+template <typename S>
+__device__ __forceinline__ void load_state(const S* base, int wave, int lane, uint4 (&raw)[StateMap<S>::STEPS]) {
+    using M = StateMap<S>;
+#pragma unroll
+    for (int j = 0; j < M::STEPS; ++j) raw[j] = ld128(base + (long long)M::row(j, wave, lane) * DK + M::key0(lane));
+}
+
+template <typename S>
+__device__ __forceinline__ void store_state(S* base, int wave, int lane,
+                                            const float (&s)[StateMap<S>::STEPS][StateGeo<S>::KPL]) {
+    using M = StateMap<S>;
+#pragma unroll
+    for (int j = 0; j < M::STEPS; ++j) st128(base + (long long)M::row(j, wave, lane) * DK + M::key0(lane), pack<S>(s[j]));
+}
+
+template <typename S>
+__device__ __forceinline__ void round_state(float (&s)[StateMap<S>::STEPS][StateGeo<S>::KPL]) {
+    using M = StateMap<S>;
+    if constexpr (M::kRound) {
+#pragma unroll
+        for (int j = 0; j < M::STEPS; ++j)
+#pragma unroll
+            for (int c = 0; c < M::KPL; ++c) s[j][c] = bfround(s[j][c]);
+    }
+}
+
+// The chain: conv + SiLU, gates, L2 norms, delta rule, read-out, gated RMSNorm, row after row
+// (reference: kda.cu:98-210, cpu.rs:410-471). The state pointers are not __restrict__: a chain may run in
+// place; each lane reads its 64 values before the first row and writes the same 64 after the last.
+// ckpt (bf16 states only): the state after every row, global row r at ckpt + r * H * 16384.
+template <typename S>
+__global__ void __launch_bounds__(THREADS) chain_kernel(
+        int H, const int32_t* __restrict__ cu_rows, int rows1,
+        const bf16_t* __restrict__ P, long long p_stride, long long b_off,
+        const bf16_t* __restrict__ A, long long a_stride, const bf16_t* __restrict__ G, long long g_stride,
+        const bf16_t* __restrict__ conv, const long long* __restrict__ conv_off, const bf16_t* __restrict__ cw,
+        const S* state_in, S* state_out, const long long* __restrict__ state_off,
+        const float* __restrict__ a_log, const float* __restrict__ dt_bias, const bf16_t* __restrict__ norm_w,
+        float eps, float lower, bf16_t* __restrict__ out, long long out_stride, S* __restrict__ ckpt,
+        float* __restrict__ k_save, bf16_t* __restrict__ v_save, float* __restrict__ g_save,
+        float* __restrict__ b_save) {
+    using M = StateMap<S>;
+    constexpr int KPL = M::KPL;
+    const long long C = 3LL * H * DK;
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+    const RowRange rr = request_rows(cu_rows, b, rows1);
+    const int rows = rr.rows;
+    const bf16_t* cs = conv + (conv_off != nullptr ? conv_off[b] : 0);
+    const long long sbase = (state_off != nullptr ? state_off[b] : 0) + (long long)h * DV * DK;
+
+    __shared__ float qs[DK], ks[DK], vs[DV], gs[DK], ys[DV];
+    __shared__ float beta_s, rinv_s;
+
+    // The state's loads go out first: their latency hides behind the first row's prologue.
+    uint4 raw[M::STEPS];
+    load_state<S>(state_in + sbase, wave, lane, raw);
+
+    const float decay_rate = expf(a_log[h]);
+    float s[M::STEPS][KPL];
+    const int key0 = M::key0(lane);
+
+    for (int r = 0; r < rows; ++r) {
+        const long long gr = rr.row0 + r;
+        // Prologue, two items per lane: lane t takes conv channel t of q|k (q for t < 128, k after), then
+        // v channel t (t < 128) or decay channel t - 128.
+#pragma unroll
+        for (int item = 0; item < 2; ++item) {
+            const bool is_conv = item == 0 || t < DK;
+            if (is_conv) {
+                const int which = item == 0 ? (t >> 7) : 2;   // 0 q, 1 k, 2 v
+                const int i = t & (DK - 1);
+                const long long c = (long long)which * H * DK + (long long)h * DK + i;
+                float acc = 0.0f;
+#pragma unroll
+                for (int tap = 0; tap < TAPS; ++tap) {
+                    const int at = r + tap;
+                    const float x = at < WINDOW ? bf2f(cs[(long long)at * C + c])
+                                                : bf2f(P[(rr.row0 + at - WINDOW) * p_stride + c]);
+                    acc = acc + bf2f(cw[c * TAPS + tap]) * x;
+                }
+                const float act = bfround(acc / (1.0f + expf(-acc)));
+                if (which == 0) qs[i] = act;
+                else if (which == 1) ks[i] = act;
+                else vs[i] = act;
+            } else {
+                const int i = t - DK;
+                const float a = bf2f(A[gr * a_stride + h * DK + i]) + dt_bias[h * DK + i];
+                gs[i] = expf(lower * sigmoidf_(decay_rate * a));
+            }
+        }
+        if (t == THREADS - 1) beta_s = bfround(sigmoidf_(bf2f(P[gr * p_stride + b_off + h])));
+        __syncthreads();
+        // L2 norms by wave 0: lanes 0..31 take q, lanes 32..63 take k.
+        if (wave == 0) {
+            float* x = lane < 32 ? qs : ks;
+            const int l32 = lane & 31;
+            float v4[4];
+            const float ss = sumsq128(x, l32, v4);
+            const float inv = 1.0f / sqrtf(ss + 1e-6f);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float y = v4[i] * inv;
+                if (lane < 32) y = y * (1.0f / sqrtf((float)DK));
+                x[l32 * 4 + i] = y;
+            }
+        }
+        __syncthreads();
+        if (r == 0) {
+#pragma unroll
+            for (int j = 0; j < M::STEPS; ++j) unpack<S>(raw[j], s[j]);
+        }
+        const float beta = beta_s;
+        float kk[KPL], qq[KPL], gg[KPL];
+#pragma unroll
+        for (int c = 0; c < KPL; ++c) {
+            kk[c] = ks[key0 + c];
+            qq[c] = qs[key0 + c];
+            gg[c] = gs[key0 + c];
+        }
+#pragma unroll
+        for (int j = 0; j < M::STEPS; ++j) {
+            const int row = M::row(j, wave, lane);
+            update_row<S>(s[j], kk, gg, vs[row], beta);
+            const float o = read_row<S>(s[j], qq);
+            if (lane % M::LPR == 0) ys[row] = bfround(o);
+        }
+        round_state<S>(s);
+        if (ckpt != nullptr) store_state<S>(ckpt + (gr * H + h) * (long long)(DV * DK), wave, lane, s);
+        if (k_save != nullptr) {
+            const long long base = (gr * H + h) * DK;
+            if (t < DK) {
+                k_save[base + t] = ks[t];
+                g_save[base + t] = gs[t];
+            } else {
+                v_save[base + t - DK] = f2bf(vs[t - DK]);
+            }
+            if (t == 0) b_save[gr * H + h] = beta;
+        }
+        __syncthreads();
+        // Gated RMSNorm (cpu.rs:361-376).
+        if (wave == 0 && lane < 32) {
+            float v4[4];
+            const float ss = sumsq128(ys, lane, v4);
+            if (lane == 0) rinv_s = 1.0f / sqrtf(ss / (float)DV + eps);
+        }
+        __syncthreads();
+        if (t < DV) {
+            const float yn = ys[t] * rinv_s;
+            const float yw = bf2f(norm_w[t]) * yn;
+            const float gate = bf2f(G[gr * g_stride + h * DV + t]);
+            out[gr * out_stride + h * DV + t] = f2bf(yw * sigmoidf_(gate));
+        }
+        __syncthreads();
+    }
+    if (state_out != nullptr) {
+        if (rows == 0) {
+#pragma unroll
+            for (int j = 0; j < M::STEPS; ++j)
+                st128(state_out + sbase + (long long)M::row(j, wave, lane) * DK + key0, raw[j]);
+        } else {
+            store_state<S>(state_out + sbase, wave, lane, s);
+        }
+    }
+}
+
+// Replay of saved rows (reference: kda.cu:214-253, cpu.rs:486-508): workgroup (layer * H + h, b). Waves are
+// independent here: every lane reads its own keys' k and exp(g) and its rows' v straight from the saves.
+template <typename S>
+__global__ void __launch_bounds__(THREADS) replay_kernel(
+        int H, const int32_t* __restrict__ cu_rows, const int32_t* __restrict__ keep, int rows1,
+        const S* state_in, S* state_out, long long state_stride, const long long* __restrict__ state_off,
+        const float* __restrict__ k_save, const bf16_t* __restrict__ v_save, const float* __restrict__ g_save,
+        const float* __restrict__ b_save, long long kv_stride, long long b_stride) {
+    using M = StateMap<S>;
+    constexpr int KPL = M::KPL;
+    const int layer = blockIdx.x / H, h = blockIdx.x % H, b = blockIdx.y;
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+    const long long row0 = cu_rows != nullptr ? cu_rows[b] : 0;
+    const int rows = keep != nullptr ? keep[b] : rows1;
+    const long long sbase = (long long)layer * state_stride + (state_off != nullptr ? state_off[b] : 0) +
+                            (long long)h * DV * DK;
+    const float* ksv = k_save + layer * kv_stride;
+    const bf16_t* vsv = v_save + layer * kv_stride;
+    const float* gsv = g_save + layer * kv_stride;
+    const float* bsv = b_save + layer * b_stride;
+    const int key0 = M::key0(lane);
+
+    uint4 raw[M::STEPS];
+    load_state<S>(state_in + sbase, wave, lane, raw);
+    if (rows <= 0) {
+#pragma unroll
+        for (int j = 0; j < M::STEPS; ++j)
+            st128(state_out + sbase + (long long)M::row(j, wave, lane) * DK + key0, raw[j]);
+        return;
+    }
+    float s[M::STEPS][KPL];
+#pragma unroll
+    for (int j = 0; j < M::STEPS; ++j) unpack<S>(raw[j], s[j]);
+    for (int r = 0; r < rows; ++r) {
+        const long long gr = row0 + r;
+        const long long base = (gr * H + h) * DK;
+        float kk[KPL], gg[KPL];
+#pragma unroll
+        for (int c = 0; c < KPL; c += 4) {
+            const float4 k4 = *reinterpret_cast<const float4*>(ksv + base + key0 + c);
+            const float4 g4 = *reinterpret_cast<const float4*>(gsv + base + key0 + c);
+            kk[c] = k4.x; kk[c + 1] = k4.y; kk[c + 2] = k4.z; kk[c + 3] = k4.w;
+            gg[c] = g4.x; gg[c + 1] = g4.y; gg[c + 2] = g4.z; gg[c + 3] = g4.w;
+        }
+        const float beta = bsv[gr * H + h];
+#pragma unroll
+        for (int j = 0; j < M::STEPS; ++j)
+            update_row<S>(s[j], kk, gg, bf2f(vsv[base + M::row(j, wave, lane)]), beta);
+        round_state<S>(s);
+    }
+    store_state<S>(state_out + sbase, wave, lane, s);
+}
+
+// Conv-window shift (reference: kda.cu:258-277, cpu.rs:512-527): lane (channel, layer, request) reads its
+// three values before writing them, so the shift runs in place.
+__global__ void conv_shift_kernel(int C, const int32_t* __restrict__ cu_rows, const int32_t* __restrict__ keep,
+                                  int keep1, bf16_t* conv, long long conv_stride,
+                                  const long long* __restrict__ conv_off, const bf16_t* P,
+                                  long long p_layer_stride, long long p_stride) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int layer = blockIdx.y, b = blockIdx.z;
+    const long long row0 = cu_rows != nullptr ? cu_rows[b] : 0;
+    const int k = keep != nullptr ? keep[b] : keep1;
+    bf16_t* win = conv + (long long)layer * conv_stride + (conv_off != nullptr ? conv_off[b] : 0);
+    const bf16_t* rows = P + (long long)layer * p_layer_stride + row0 * p_stride;
+    bf16_t v[WINDOW];
+#pragma unroll
+    for (int j = 0; j < WINDOW; ++j) {
+        const long long src = (long long)k + j;
+        v[j] = src < WINDOW ? win[src * C + c] : rows[(src - WINDOW) * p_stride + c];
+    }
+#pragma unroll
+    for (int j = 0; j < WINDOW; ++j) win[(long long)j * C + c] = v[j];
+}
+
+// Commit by selection: workgroup (layer * H + h, b) copies one head of the checkpoint after row keep[b] - 1.
+__global__ void __launch_bounds__(THREADS) select_kernel(
+        int H, const int32_t* __restrict__ cu_rows, const int32_t* __restrict__ keep,
+        const bf16_t* __restrict__ ckpt, long long ckpt_layer_stride, bf16_t* __restrict__ state,
+        long long state_stride, const long long* __restrict__ state_off) {
+    const int layer = blockIdx.x / H, h = blockIdx.x % H, b = blockIdx.y;
+    const int k = keep[b];
+    if (k <= 0) return;
+    const long long gr = (long long)cu_rows[b] + k - 1;
+    const bf16_t* src = ckpt + (long long)layer * ckpt_layer_stride + (gr * H + h) * (long long)(DV * DK);
+    bf16_t* dst = state + (long long)layer * state_stride + state_off[b] + (long long)h * DV * DK;
+    uint4 v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = ld128(src + (i * THREADS + threadIdx.x) * 8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) st128(dst + (i * THREADS + threadIdx.x) * 8, v[i]);
+}
+
+inline int launched() { return (int)hipGetLastError(); }
+
+// States, checkpoints and saves move in 128-bit pieces: their base pointers must be 16-byte aligned (and the
+// device-side offsets multiples of 8 elements, which whole heads always are).
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline const bf16_t* bfp(const glm53f_bf16* x) { return reinterpret_cast<const bf16_t*>(x); }
+inline bf16_t* bfp(glm53f_bf16* x) { return reinterpret_cast<bf16_t*>(x); }
+
+// Host-side checks shared by the chain entry points (reference: kda.cu:290-299).
+inline bool chain_args_ok(int32_t heads, const void* p, const void* a, const void* g, const void* conv,
+                          const void* conv_w, const void* state_in, const void* a_log, const void* dt_bias,
+                          const void* norm_w, const void* out, const void* k_save, const void* v_save,
+                          const void* g_save, const void* b_save) {
+    if (heads < 1 || heads > 65535) return false;
+    if (!p || !a || !g || !conv || !conv_w || !state_in || !a_log || !dt_bias || !norm_w || !out) return false;
+    const int saves = (k_save != nullptr) + (v_save != nullptr) + (g_save != nullptr) + (b_save != nullptr);
+    return saves == 0 || saves == 4;
+}
+
+template <typename S>
+int chain_batch_launch(int32_t heads, int32_t batch, const int32_t* cu_rows, const glm53f_bf16* p, int64_t p_stride,
+                       int64_t b_off, const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g, int64_t g_stride,
+                       const glm53f_bf16* conv, const int64_t* conv_off, const glm53f_bf16* conv_w, const S* state_in,
+                       S* state_out, const int64_t* state_off, const float* a_log, const float* dt_bias,
+                       const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out, int64_t out_stride,
+                       S* ckpt, float* k_save, glm53f_bf16* v_save, float* g_save, float* b_save,
+                       glm53f_stream_t stream) {
+    if (batch < 1 || batch > 65535 || !cu_rows || !conv_off || !state_off ||
+        !chain_args_ok(heads, p, a, g, conv, conv_w, state_in, a_log, dt_bias, norm_w, out, k_save, v_save, g_save,
+                       b_save))
+        return kInvalid;
+    if (!aligned16(state_in) || !aligned16(state_out) || !aligned16(ckpt)) return kInvalid;
+    chain_kernel<S><<<dim3(heads, batch), THREADS, 0, (hipStream_t)stream>>>(
+        heads, cu_rows, 0, bfp(p), p_stride, b_off, bfp(a), a_stride, bfp(g), g_stride, bfp(conv),
+        reinterpret_cast<const long long*>(conv_off), bfp(conv_w), state_in, state_out,
+        reinterpret_cast<const long long*>(state_off), a_log, dt_bias, bfp(norm_w), eps, lower, bfp(out), out_stride,
+        ckpt, k_save, bfp(v_save), g_save, b_save);
+    return launched();
+}
+
+// Host-side checks of the replays (reference: kda.cu:376-388).
+template <typename S>
+int replay_launch(int32_t heads, int32_t layers, int32_t batch, const int32_t* cu_rows, const int32_t* keep,
+                  int32_t rows, const S* state_in, S* state_out, int64_t state_stride, const int64_t* state_off,
+                  const float* k_save, const glm53f_bf16* v_save, const float* g_save, const float* b_save,
+                  int64_t kv_stride, int64_t b_stride, glm53f_stream_t stream) {
+    if (heads < 1 || layers < 1 || batch < 1 || batch > 65535 || (long long)heads * layers > 0x7fffffffLL ||
+        !state_in || !state_out || !k_save || !v_save || !g_save || !b_save || rows < 0)
+        return kInvalid;
+    if (!aligned16(state_in) || !aligned16(state_out) || !aligned16(k_save) || !aligned16(g_save) ||
+        (kv_stride & 3) != 0)
+        return kInvalid;
+    replay_kernel<S><<<dim3(heads * layers, batch), THREADS, 0, (hipStream_t)stream>>>(
+        heads, cu_rows, keep, rows, state_in, state_out, state_stride,
+        reinterpret_cast<const long long*>(state_off), k_save, bfp(v_save), g_save, b_save, kv_stride, b_stride);
+    return launched();
+}
+
+constexpr int kShiftThreads = 256;
+
+// Host-side checks of the conv shift (reference: kda.cu:433-444).
+inline int conv_shift_launch(int32_t channels, int32_t layers, int32_t batch, const int32_t* cu_rows,
+                             const int32_t* keep, int32_t keep1, glm53f_bf16* conv, int64_t conv_stride,
+                             const int64_t* conv_off, const glm53f_bf16* p, int64_t p_layer_stride, int64_t p_stride,
+                             glm53f_stream_t stream) {
+    if (channels < 1 || layers < 1 || layers > 65535 || batch < 1 || batch > 65535 || !conv || !p || keep1 < 0)
+        return kInvalid;
+    const dim3 grid((channels + kShiftThreads - 1) / kShiftThreads, layers, batch);
+    conv_shift_kernel<<<grid, kShiftThreads, 0, (hipStream_t)stream>>>(
+        channels, cu_rows, keep, keep1, bfp(conv), conv_stride, reinterpret_cast<const long long*>(conv_off), bfp(p),
+        p_layer_stride, p_stride);
+    return launched();
+}
+
+}  // namespace
+}  // namespace kda
+
+using namespace kda;
+
+extern "C" int glm53f_kda_chain(int32_t heads, int32_t rows, const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
+                                const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g, int64_t g_stride,
+                                const glm53f_bf16* conv, const glm53f_bf16* conv_w, const float* state_in,
+                                float* state_out, const float* a_log, const float* dt_bias,
+                                const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out,
+                                int64_t out_stride, float* k_save, glm53f_bf16* v_save, float* g_save,
+                                float* b_save, glm53f_stream_t stream) {
+    if (rows < 1 || !chain_args_ok(heads, p, a, g, conv, conv_w, state_in, a_log, dt_bias, norm_w, out, k_save,
+                                   v_save, g_save, b_save))
+        return kInvalid;
+    if (!aligned16(state_in) || !aligned16(state_out)) return kInvalid;
+    chain_kernel<float><<<dim3(heads, 1), THREADS, 0, (hipStream_t)stream>>>(
+        heads, nullptr, rows, bfp(p), p_stride, b_off, bfp(a), a_stride, bfp(g), g_stride, bfp(conv), nullptr,
+        bfp(conv_w), state_in, state_out, nullptr, a_log, dt_bias, bfp(norm_w), eps, lower, bfp(out), out_stride,
+        nullptr, k_save, bfp(v_save), g_save, b_save);
+    return launched();
+}
+
+extern "C" int glm53f_kda_chain_batch(int32_t heads, int32_t batch, const int32_t* cu_rows, const glm53f_bf16* p,
+                                      int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride,
+                                      const glm53f_bf16* g, int64_t g_stride, const glm53f_bf16* conv,
+                                      const int64_t* conv_off, const glm53f_bf16* conv_w, const float* state_in,
+                                      float* state_out, const int64_t* state_off, const float* a_log,
+                                      const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower,
+                                      glm53f_bf16* out, int64_t out_stride, float* k_save, glm53f_bf16* v_save,
+                                      float* g_save, float* b_save, glm53f_stream_t stream) {
+    return chain_batch_launch<float>(heads, batch, cu_rows, p, p_stride, b_off, a, a_stride, g, g_stride, conv,
+                                     conv_off, conv_w, state_in, state_out, state_off, a_log, dt_bias, norm_w, eps,
+                                     lower, out, out_stride, nullptr, k_save, v_save, g_save, b_save, stream);
+}
+
+extern "C" int glm53f_kda_chain_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,
+                                                const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
+                                                const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g,
+                                                int64_t g_stride, const glm53f_bf16* conv, const int64_t* conv_off,
+                                                const glm53f_bf16* conv_w, const glm53f_bf16* state_in,
+                                                glm53f_bf16* state_out, const int64_t* state_off,
+                                                const float* a_log, const float* dt_bias,
+                                                const glm53f_bf16* norm_w, float eps, float lower,
+                                                glm53f_bf16* out, int64_t out_stride, float* k_save,
+                                                glm53f_bf16* v_save, float* g_save, float* b_save,
+                                                glm53f_stream_t stream) {
+    return chain_batch_launch<bf16_t>(heads, batch, cu_rows, p, p_stride, b_off, a, a_stride, g, g_stride, conv,
+                                      conv_off, conv_w, bfp(state_in), bfp(state_out), state_off, a_log, dt_bias,
+                                      norm_w, eps, lower, out, out_stride, nullptr, k_save, v_save, g_save, b_save,
+                                      stream);
+}
+
+extern "C" int glm53f_kda_verify_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,
+                                                 const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
+                                                 const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g,
+                                                 int64_t g_stride, const glm53f_bf16* conv, const int64_t* conv_off,
+                                                 const glm53f_bf16* conv_w, const glm53f_bf16* state_in,
+                                                 const int64_t* state_off, const float* a_log,
+                                                 const float* dt_bias, const glm53f_bf16* norm_w, float eps,
+                                                 float lower, glm53f_bf16* out, int64_t out_stride,
+                                                 glm53f_bf16* ckpt, float* k_save, glm53f_bf16* v_save,
+                                                 float* g_save, float* b_save, glm53f_stream_t stream) {
+    if (!ckpt) return kInvalid;
+    return chain_batch_launch<bf16_t>(heads, batch, cu_rows, p, p_stride, b_off, a, a_stride, g, g_stride, conv,
+                                      conv_off, conv_w, bfp(state_in), nullptr, state_off, a_log, dt_bias, norm_w,
+                                      eps, lower, out, out_stride, bfp(ckpt), k_save, v_save, g_save, b_save, stream);
+}
+
+extern "C" int glm53f_kda_select_batch_bf16state(int32_t heads, int32_t layers, int32_t batch,
+                                                 const int32_t* cu_rows, const int32_t* keep,
+                                                 const glm53f_bf16* ckpt, int64_t ckpt_layer_stride,
+                                                 glm53f_bf16* state, int64_t state_stride,
+                                                 const int64_t* state_off, glm53f_stream_t stream) {
+    if (heads < 1 || layers < 1 || batch < 1 || batch > 65535 || (long long)heads * layers > 0x7fffffffLL ||
+        !cu_rows || !keep || !ckpt || !state || !state_off || !aligned16(ckpt) || !aligned16(state) ||
+        (ckpt_layer_stride & 7) != 0 || (state_stride & 7) != 0)
+        return kInvalid;
+    select_kernel<<<dim3(heads * layers, batch), THREADS, 0, (hipStream_t)stream>>>(
+        heads, cu_rows, keep, bfp(ckpt), ckpt_layer_stride, bfp(state), state_stride,
+        reinterpret_cast<const long long*>(state_off));
+    return launched();
+}
+
+extern "C" int glm53f_kda_replay(int32_t heads, int32_t rows, const float* state_in, float* state_out,
+                                 const float* k_save, const glm53f_bf16* v_save, const float* g_save,
+                                 const float* b_save, glm53f_stream_t stream) {
+    return replay_launch<float>(heads, 1, 1, nullptr, nullptr, rows, state_in, state_out, 0, nullptr, k_save, v_save,
+                                g_save, b_save, 0, 0, stream);
+}
+
+extern "C" int glm53f_kda_replay_layers(int32_t heads, int32_t layers, int32_t rows, const float* state_in,
+                                        float* state_out, int64_t state_stride, const float* k_save,
+                                        const glm53f_bf16* v_save, const float* g_save, const float* b_save,
+                                        int64_t kv_stride, int64_t b_stride, glm53f_stream_t stream) {
+    return replay_launch<float>(heads, layers, 1, nullptr, nullptr, rows, state_in, state_out, state_stride, nullptr,
+                                k_save, v_save, g_save, b_save, kv_stride, b_stride, stream);
+}
+
+extern "C" int glm53f_kda_replay_batch(int32_t heads, int32_t layers, int32_t batch, const int32_t* cu_rows,
+                                       const int32_t* keep, const float* state_in, float* state_out,
+                                       int64_t state_stride, const int64_t* state_off, const float* k_save,
+                                       const glm53f_bf16* v_save, const float* g_save, const float* b_save,
+                                       int64_t kv_stride, int64_t b_stride, glm53f_stream_t stream) {
+    if (!cu_rows || !keep || !state_off) return kInvalid;
+    return replay_launch<float>(heads, layers, batch, cu_rows, keep, 0, state_in, state_out, state_stride, state_off,
+                                k_save, v_save, g_save, b_save, kv_stride, b_stride, stream);
+}
+
+extern "C" int glm53f_kda_replay_batch_bf16state(int32_t heads, int32_t layers, int32_t batch,
+                                                 const int32_t* cu_rows, const int32_t* keep,
+                                                 const glm53f_bf16* state_in, glm53f_bf16* state_out,
+                                                 int64_t state_stride, const int64_t* state_off,
+                                                 const float* k_save, const glm53f_bf16* v_save,
+                                                 const float* g_save, const float* b_save, int64_t kv_stride,
+                                                 int64_t b_stride, glm53f_stream_t stream) {
+    if (!cu_rows || !keep || !state_off) return kInvalid;
+    return replay_launch<bf16_t>(heads, layers, batch, cu_rows, keep, 0, bfp(state_in), bfp(state_out), state_stride,
+                                 state_off, k_save, v_save, g_save, b_save, kv_stride, b_stride, stream);
+}
+
+extern "C" int glm53f_kda_conv_shift(int32_t channels, int32_t keep, glm53f_bf16* conv, const glm53f_bf16* p,
+                                     int64_t p_stride, glm53f_stream_t stream) {
+    return conv_shift_launch(channels, 1, 1, nullptr, nullptr, keep, conv, 0, nullptr, p, 0, p_stride, stream);
+}
+
+extern "C" int glm53f_kda_conv_shift_batch(int32_t channels, int32_t layers, int32_t batch, const int32_t* cu_rows,
+                                           const int32_t* keep, glm53f_bf16* conv, int64_t conv_stride,
+                                           const int64_t* conv_off, const glm53f_bf16* p, int64_t p_layer_stride,
+                                           int64_t p_stride, glm53f_stream_t stream) {
+    if (!cu_rows || !keep || !conv_off) return kInvalid;
+    return conv_shift_launch(channels, layers, batch, cu_rows, keep, 0, conv, conv_stride, conv_off, p,
+                             p_layer_stride, p_stride, stream);
+}
+
+extern "C" const char* glm53f_kda_arch(void) { return "gfx950"; }

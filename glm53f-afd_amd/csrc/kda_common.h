@@ -1,0 +1,179 @@
+// Shared device helpers of the KDA kernels (gfx950, wave64).
+#ifndef GLM53F_KDA_COMMON_H
+#define GLM53F_KDA_COMMON_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "glm53f_kda.h"
+
+namespace kda {
+
+constexpr int DK = 128, DV = 128, TAPS = 4, WINDOW = 3;
+constexpr int kInvalid = 1;  // hipErrorInvalidValue
+
+typedef uint16_t bf16_t;
+
+__device__ __forceinline__ float bf2f(bf16_t b) { return __uint_as_float((uint32_t)b << 16); }
+
+// Round to nearest even, NaN quieted: the bits of the reference's bf16::from_f32 (src/bf16.rs:6-13).
+__device__ __forceinline__ bf16_t f2bf(float x) {
+    const uint32_t u = __float_as_uint(x);
+    if (x != x) return (bf16_t)((u >> 16) | 0x0040u);
+    return (bf16_t)((u + (0x7fffu + ((u >> 16) & 1u))) >> 16);
+}
+
+__device__ __forceinline__ float bfround(float x) { return bf2f(f2bf(x)); }
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// Request b's global rows: [row0, row0 + rows). Without cu_rows: one request of rows1 rows.
+struct RowRange {
+    long long row0;
+    int rows;
+};
+
+__device__ __forceinline__ RowRange request_rows(const int32_t* cu_rows, int b, int rows1) {
+    if (cu_rows == nullptr) return {0, rows1};
+    const int r0 = cu_rows[b];
+    return {(long long)r0, cu_rows[b + 1] - r0};
+}
+
+// How a state element type maps onto a workgroup of 256 lanes (4 waves). Every lane moves 128 bits per
+// access: KPL consecutive keys of one value row. LPR lanes share a value row, a wave covers RPW rows per
+// step and the workgroup 4 * RPW; STEPS steps cover the 128 value rows, 64 state values per lane.
+template <typename S>
+struct StateGeo;
+template <>
+struct StateGeo<float> {
+    static constexpr int KPL = 4;
+};
+template <>
+struct StateGeo<bf16_t> {
+    static constexpr int KPL = 8;
+};
+
+template <typename S>
+struct StateMap {
+    static constexpr int KPL = StateGeo<S>::KPL;
+    static constexpr int NP = KPL / 4;         // partial sums per lane (groups of 4 consecutive keys)
+    static constexpr int LPR = DK / KPL;       // lanes per value row
+    static constexpr int RPW = 64 / LPR;       // value rows per wave per step
+    static constexpr int RPS = 4 * RPW;        // value rows per workgroup per step
+    static constexpr int STEPS = DV / RPS;
+    static constexpr bool kRound = sizeof(S) == 2;
+
+    // Value row of step j for this lane, and its first key.
+    static __device__ __forceinline__ int row(int j, int wave, int lane) { return j * RPS + wave * RPW + lane / LPR; }
+    static __device__ __forceinline__ int key0(int lane) { return (lane % LPR) * KPL; }
+};
+
+// 128-bit raw state access.
+__device__ __forceinline__ uint4 ld128(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ void st128(void* p, uint4 v) { *reinterpret_cast<uint4*>(p) = v; }
+
+template <typename S>
+__device__ __forceinline__ void unpack(const uint4 raw, float (&s)[StateGeo<S>::KPL]);
+template <>
+__device__ __forceinline__ void unpack<float>(const uint4 raw, float (&s)[4]) {
+    s[0] = __uint_as_float(raw.x);
+    s[1] = __uint_as_float(raw.y);
+    s[2] = __uint_as_float(raw.z);
+    s[3] = __uint_as_float(raw.w);
+}
+template <>
+__device__ __forceinline__ void unpack<bf16_t>(const uint4 raw, float (&s)[8]) {
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        s[2 * i] = __uint_as_float(w[i] << 16);
+        s[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+
+// Pack for the store. A bf16 state is already bf16-exact here (rounded after every row, or just loaded),
+// so the conversion rounds nothing.
+template <typename S>
+__device__ __forceinline__ uint4 pack(const float (&s)[StateGeo<S>::KPL]);
+template <>
+__device__ __forceinline__ uint4 pack<float>(const float (&s)[4]) {
+    return make_uint4(__float_as_uint(s[0]), __float_as_uint(s[1]), __float_as_uint(s[2]), __float_as_uint(s[3]));
+}
+template <>
+__device__ __forceinline__ uint4 pack<bf16_t>(const float (&s)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f2bf(s[2 * i]) | ((uint32_t)f2bf(s[2 * i + 1]) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// The sum over one value row's 128 keys of per-lane partial sums, in the order of the reference's CPU
+// model (cpu.rs:214-239): partial l (l = 0..31) covers keys 4l..4l+3, then an xor butterfly over l with
+// offsets 16, 8, 4, 2, 1. With NP partials per lane the low bits of l live inside the lane, so the
+// butterfly's first steps cross lanes and its last adds the lane's own partials. Every lane of the row
+// ends with the same bits.
+template <int NP, int LPR>
+__device__ __forceinline__ float row_sum(float (&x)[NP]) {
+#pragma unroll
+    for (int m = LPR / 2; m >= 1; m >>= 1) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) x[p] = x[p] + __shfl_xor(x[p], m, 64);
+    }
+    if (NP == 2) return x[0] + x[1];
+    return x[0];
+}
+
+// One delta-rule step on this lane's KPL keys of one value row: the arithmetic, operation for operation,
+// of the reference's `update` (cpu.rs:324-344, kda.cu:38-53). No fused multiply-add (the file is compiled
+// with contraction off).
+template <typename S>
+__device__ __forceinline__ void update_row(float (&s)[StateGeo<S>::KPL], const float (&kk)[StateGeo<S>::KPL],
+                                           const float (&gg)[StateGeo<S>::KPL], float v, float beta) {
+    using M = StateMap<S>;
+    float part[M::NP];
+#pragma unroll
+    for (int p = 0; p < M::NP; ++p) {
+        float kv = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = 4 * p + i;
+            s[c] = s[c] * gg[c];
+            kv = kv + s[c] * kk[c];
+        }
+        part[p] = kv;
+    }
+    const float kv = row_sum<M::NP, M::LPR>(part);
+    const float delta = (v - kv) * beta;
+#pragma unroll
+    for (int c = 0; c < M::KPL; ++c) s[c] = s[c] + kk[c] * delta;
+}
+
+// The read-out of one value row (cpu.rs:347-353), not rounded.
+template <typename S>
+__device__ __forceinline__ float read_row(const float (&s)[StateGeo<S>::KPL], const float (&qq)[StateGeo<S>::KPL]) {
+    using M = StateMap<S>;
+    float part[M::NP];
+#pragma unroll
+    for (int p = 0; p < M::NP; ++p) {
+        float o = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o = o + s[4 * p + i] * qq[4 * p + i];
+        part[p] = o;
+    }
+    return row_sum<M::NP, M::LPR>(part);
+}
+
+// dot128 (cpu.rs:229-239) of an LDS vector with itself, by the 32 lanes of a half wave (lane32 = 0..31).
+__device__ __forceinline__ float sumsq128(const float* x, int lane32, float (&v4)[4]) {
+    float part[1] = {0.0f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v4[i] = x[lane32 * 4 + i];
+        part[0] = part[0] + v4[i] * v4[i];
+    }
+    return row_sum<1, 32>(part);
+}
+
+}  // namespace kda
+
+#endif  // GLM53F_KDA_COMMON_H
