@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the KDA hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify]
+
+Prints ONE JSON line. The headline `value` is the decode step's state traffic in GB/s at BASELINE config 1
+(16 slots x 1 token out of a 48-slot bf16 pool, 64 heads, 34 layers each with its own pool so the working set
+exceeds the last-level cache); a "step" is one decode step over the 34 KDA layers (chain + conv shift per
+layer). The same line carries the chunked prefill (config 2: T = 8192 as four sequential 2048-row calls on one
+slot) and the checkpointing verify (config 4: 48 slots x 16 drafts) under `prefill` and `verify`, each with its
+own roofline object, and the CPU oracle timed on this host's cores as `cpu_baseline`.
+
+Inputs are synthetic with BASELINE's distributions, generated on the GPU; all buffers are resident in HBM
+before the timed region. Kernel durations are measured with events on the stream the kernels are launched on.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "glm53f-afd_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+import numpy as np
+import torch
+
+from glm53f_kda import DK, DV, HEADS, LAYERS, WINDOW, channels, ffi, state_len
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
+DEV = "cuda:0"
+
+METRIC = "KDA prefill tok/s per layer at T=8K (MFMA %); decode state GB/s at 16 slots"
+
+
+def ptr(t, off=0):
+    return None if t is None else t.data_ptr() + off * t.element_size()
+
+
+class Layer:
+    """Random-init weights of one KDA layer with BASELINE's gate mapping: A_log = 0, dt_bias = 0, so
+    g = -5 * sigmoid(a) and a = logit(softplus(z) / 5) gives g = -softplus(z)."""
+
+    def __init__(self, heads, gen):
+        c = channels(heads)
+        self.heads = heads
+        self.conv_w = ((torch.rand(c * 4, device=DEV, generator=gen) - 0.5) * 1.2).to(torch.bfloat16)
+        self.a_log = torch.zeros(heads, device=DEV)
+        self.dt_bias = torch.zeros(heads * DK, device=DEV)
+        self.norm_w = torch.ones(DV, device=DEV, dtype=torch.bfloat16)
+        self.eps, self.lower = 1e-5, -5.0
+
+    def args(self):
+        return [ptr(self.a_log), ptr(self.dt_bias), ptr(self.norm_w), self.eps, self.lower]
+
+
+class RowBuffers:
+    """Projection rows in the engine's layout: p rows of C + H columns (beta logits behind q|k|v), dense a, g,
+    out (reference call site: crates/glm53f-forward/src/forward.rs:3672-3705)."""
+
+    def __init__(self, heads, rows, gen):
+        c = channels(heads)
+        self.heads, self.rows = heads, rows
+        self.p_stride = c + heads
+        self.p = torch.randn(rows, self.p_stride, device=DEV, generator=gen).to(torch.bfloat16)
+        z = torch.randn(rows, heads * DK, device=DEV, generator=gen, dtype=torch.float64)
+        sp = torch.clamp(torch.nn.functional.softplus(z), max=4.999)
+        self.a = (torch.log(sp / 5.0) - torch.log1p(-sp / 5.0)).to(torch.bfloat16)
+        self.g = torch.randn(rows, heads * DV, device=DEV, generator=gen).to(torch.bfloat16)
+        self.out = torch.zeros(rows, heads * DV, device=DEV, dtype=torch.bfloat16)
+
+    def row_args(self, first=0):
+        c = channels(self.heads)
+        return [ptr(self.p, first * self.p_stride), self.p_stride, c, ptr(self.a, first * self.heads * DK),
+                self.heads * DK, ptr(self.g, first * self.heads * DV), self.heads * DV]
+
+    def out_args(self, first=0):
+        return [ptr(self.out, first * self.heads * DV), self.heads * DV]
+
+    def to_oracle(self, o, first, n):
+        c, h = channels(self.heads), self.heads
+        f = lambda t: t.float().cpu().numpy().reshape(-1)
+        return o.Rows(h, n, f(self.p[first:first + n, :c]), f(self.a[first:first + n]),
+                      f(self.p[first:first + n, c:c + h]), f(self.g[first:first + n]))
+
+
+def timed(fn, steps, warmup, stream):
+    """W untimed calls, then exactly K timed ones between events on `stream`; returns ms per call."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(steps):
+        fn()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def check(code, what):
+    if code != 0:
+        raise RuntimeError(f"{what} returned {code}")
+
+
+# ------------------------------------------------------------------------------------------------ decode
+
+def bench_decode(steps, warmup, stream, cpu=True):
+    heads, slots_n, batch, layers = HEADS, 48, 16, LAYERS
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    layer = Layer(heads, gen)
+    n, cw = state_len(heads), WINDOW * channels(heads)
+    # One pool per layer, as the engine lays them out: 34 x 48 x 2 MiB of bf16 state.
+    pools = (torch.randn(layers, slots_n * n, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
+    convs = torch.randn(layers, slots_n * cw, device=DEV, generator=gen).to(torch.bfloat16)
+    rows = RowBuffers(heads, batch, gen)
+    perm = torch.randperm(slots_n, generator=torch.Generator().manual_seed(2))[:batch]
+    cu = torch.arange(batch + 1, dtype=torch.int32, device=DEV)
+    keep = torch.ones(batch, dtype=torch.int32, device=DEV)
+    soff = (perm.to(torch.int64) * n).to(DEV)
+    coff = (perm.to(torch.int64) * cw).to(DEV)
+    st = stream.cuda_stream
+    c = channels(heads)
+
+    # Argument lists are built once: the timed loops only make the C calls.
+    chain_fn, shift_fn = ffi.glm53f_kda_chain_batch_bf16state, ffi.glm53f_kda_conv_shift_batch
+    chain_args = [(heads, batch, ptr(cu), *rows.row_args(), ptr(convs[l]), ptr(coff), ptr(layer.conv_w),
+                   ptr(pools[l]), ptr(pools[l]), ptr(soff), *layer.args(), *rows.out_args(), None, None, None, None,
+                   st) for l in range(layers)]
+    shift_args = [(c, 1, batch, ptr(cu), ptr(keep), ptr(convs[l]), 0, ptr(coff), ptr(rows.p), 0, rows.p_stride, st)
+                  for l in range(layers)]
+
+    def chain(l):
+        check(chain_fn(*chain_args[l]), "chain")
+
+    def shift(l):
+        check(shift_fn(*shift_args[l]), "conv_shift")
+
+    def step():
+        for l in range(layers):
+            chain(l)
+            shift(l)
+
+    def chains_only():
+        for l in range(layers):
+            chain(l)
+
+    ms_step = timed(step, steps, warmup, stream)
+    ms_chain = timed(chains_only, steps, max(1, warmup // 2), stream) / layers
+    state_bytes = 2 * batch * n * 2                      # read + write of 16 bf16 states: 67,108,864 B
+    res = {
+        "ms_per_step": ms_step,
+        "state_GBps": layers * state_bytes / (ms_step * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": state_bytes / (ms_chain * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": state_bytes / (ms_chain * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "chain_kernel<bf16>", "bytes_per_launch": state_bytes,
+                     "us_per_launch": ms_chain * 1e3},
+    }
+    if cpu:
+        from oracle import kda_oracle as o
+        threads = min(16, os.cpu_count() or 1)
+        p = o.LayerParams(heads, layer.conv_w.float().cpu().numpy(), layer.a_log.cpu().numpy(),
+                          layer.dt_bias.cpu().numpy(), layer.norm_w.float().cpu().numpy())
+        reqs = [rows.to_oracle(o, i, 1) for i in range(batch)]
+        pool0 = pools[0].float().cpu().numpy()
+        conv0 = convs[0].float().cpu().numpy()
+        slots = perm.tolist()
+
+        def one_layer_step():
+            for i, s in enumerate(slots):
+                o.chain_bf16_state(p, conv0[s * cw:(s + 1) * cw], pool0[s * n:(s + 1) * n], reqs[i], threads=threads)
+
+        one_layer_step()
+        t0, reps = time.perf_counter(), 0
+        while time.perf_counter() - t0 < 3.0:
+            one_layer_step()
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": state_bytes / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                               "sample": f"config 1 in full for one layer (16 slots x 64 heads x 1 row, bf16-rounded "
+                                         f"state), {reps} repetitions of the C oracle chain_bf16_state, "
+                                         f"{dt * 1e3:.2f} ms per layer-step"}
+    return res
+
+
+# ------------------------------------------------------------------------------------------------ main
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", choices=["decode", "prefill", "verify"], default=None)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; the KDA path shards by heads or slots with no exchange step, "
+              "and no multi-GPU figure is produced. Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    ffi.lib()
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream()
+    line = {"metric": METRIC, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32 (bf16 state and rows)",
+            "data": "synthetic"}
+    dec = None
+    if args.only in (None, "decode"):
+        dec = bench_decode(args.steps, args.warmup, stream, cpu=not args.no_cpu)
+        line.update({"value": dec["state_GBps"], "ms_per_step": dec["ms_per_step"], "roofline": dec["roofline"],
+                     "config": {"workload": "BASELINE config 1: decode, 16 slots x 1 token of a 48-slot bf16 pool, "
+                                            "H=64, dk=dv=128, 34 layers (one pool each), chain + conv shift per layer",
+                                "slots": 16, "pool_slots": 48, "heads": 64, "layers": 34}})
+        if "cpu_baseline" in dec:
+            line["cpu_baseline"] = dec["cpu_baseline"]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -14,30 +14,26 @@ namespace {
 
 constexpr int THREADS = 256;
 
+// State access: a uniform base (bumped per step by a constant, scalar arithmetic) plus one 32-bit lane offset,
+// so no per-step 64-bit lane addresses are kept alive.
 template <typename S>
-__device__ __forceinline__ void load_state(const S* base, int wave, int lane, uint4 (&raw)[StateMap<S>::STEPS]) {
+__device__ __forceinline__ unsigned lane_offset(int wave, int lane) {
     using M = StateMap<S>;
-#pragma unroll
-    for (int j = 0; j < M::STEPS; ++j) raw[j] = ld128(base + (long long)M::row(j, wave, lane) * DK + M::key0(lane));
+    return (unsigned)(M::row(0, wave, lane) * DK + M::key0(lane));
 }
 
 template <typename S>
-__device__ __forceinline__ void store_state(S* base, int wave, int lane,
-                                            const float (&s)[StateMap<S>::STEPS][StateGeo<S>::KPL]) {
+__device__ __forceinline__ void load_state(const S* base, unsigned off, uint4 (&raw)[StateMap<S>::STEPS]) {
     using M = StateMap<S>;
 #pragma unroll
-    for (int j = 0; j < M::STEPS; ++j) st128(base + (long long)M::row(j, wave, lane) * DK + M::key0(lane), pack<S>(s[j]));
+    for (int j = 0; j < M::STEPS; ++j) raw[j] = ld128((base + j * M::RPS * DK) + off);
 }
 
 template <typename S>
-__device__ __forceinline__ void round_state(float (&s)[StateMap<S>::STEPS][StateGeo<S>::KPL]) {
+__device__ __forceinline__ void store_raw(S* base, unsigned off, const uint4 (&raw)[StateMap<S>::STEPS]) {
     using M = StateMap<S>;
-    if constexpr (M::kRound) {
 #pragma unroll
-        for (int j = 0; j < M::STEPS; ++j)
-#pragma unroll
-            for (int c = 0; c < M::KPL; ++c) s[j][c] = bfround(s[j][c]);
-    }
+    for (int j = 0; j < M::STEPS; ++j) st128((base + j * M::RPS * DK) + off, raw[j]);
 }
 
 // The chain: conv + SiLU, gates, L2 norms, delta rule, read-out, gated RMSNorm, row after row
@@ -45,7 +41,7 @@ __device__ __forceinline__ void round_state(float (&s)[StateMap<S>::STEPS][State
 // place; each lane reads its 64 values before the first row and writes the same 64 after the last.
 // ckpt (bf16 states only): the state after every row, global row r at ckpt + r * H * 16384.
 template <typename S>
-__global__ void __launch_bounds__(THREADS) chain_kernel(
+__global__ void __launch_bounds__(THREADS, 4) chain_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1,
         const bf16_t* __restrict__ P, long long p_stride, long long b_off,
         const bf16_t* __restrict__ A, long long a_stride, const bf16_t* __restrict__ G, long long g_stride,
@@ -68,48 +64,60 @@ __global__ void __launch_bounds__(THREADS) chain_kernel(
     __shared__ float qs[DK], ks[DK], vs[DV], gs[DK], ys[DV];
     __shared__ float beta_s, rinv_s;
 
-    // The state's loads go out first: their latency hides behind the first row's prologue.
-    uint4 raw[M::STEPS];
-    load_state<S>(state_in + sbase, wave, lane, raw);
-
-    const float decay_rate = expf(a_log[h]);
-    float s[M::STEPS][KPL];
+    const unsigned soff_lane = lane_offset<S>(wave, lane);
     const int key0 = M::key0(lane);
+    if (rows <= 0) {
+        // A request without rows: its state is copied (with loads of its own, so that this path shares no
+        // registers with the main one).
+        if (state_out != nullptr && state_out != state_in) {
+            uint4 cp[M::STEPS];
+            load_state<S>(state_in + sbase, soff_lane, cp);
+            store_raw<S>(state_out + sbase, soff_lane, cp);
+        }
+        return;
+    }
+    // The state's loads go out first: their latency hides behind the first row's prologue. Between rows the
+    // state stays in its stored form (`raw`: packed bf16 pairs, or f32 bits): a bf16 state is rounded after
+    // every row anyway, and the packed form halves the registers it holds.
+    uint4 raw[M::STEPS];
+    load_state<S>(state_in + sbase, soff_lane, raw);
+    const float decay_rate = expf(a_log[h]);
 
-    for (int r = 0; r < rows; ++r) {
+    // A row's prologue, two items per lane: lane t takes conv channel t of q|k (q for t < 128, k after), then
+    // v channel t (t < 128) or decay channel t - 128; then the L2 norms of q and k by wave 0.
+    auto prologue = [&](int r) {
         const long long gr = rr.row0 + r;
-        // Prologue, two items per lane: lane t takes conv channel t of q|k (q for t < 128, k after), then
-        // v channel t (t < 128) or decay channel t - 128.
 #pragma unroll
         for (int item = 0; item < 2; ++item) {
             const bool is_conv = item == 0 || t < DK;
             if (is_conv) {
                 const int which = item == 0 ? (t >> 7) : 2;   // 0 q, 1 k, 2 v
                 const int i = t & (DK - 1);
-                const long long c = (long long)which * H * DK + (long long)h * DK + i;
+                const unsigned c = (unsigned)(which * H * DK + h * DK + i);
+                const uint2 w4 = *reinterpret_cast<const uint2*>(cw + (size_t)c * TAPS);   // the 4 taps
+                const float wt[TAPS] = {__uint_as_float(w4.x << 16), __uint_as_float(w4.x & 0xffff0000u),
+                                        __uint_as_float(w4.y << 16), __uint_as_float(w4.y & 0xffff0000u)};
                 float acc = 0.0f;
 #pragma unroll
                 for (int tap = 0; tap < TAPS; ++tap) {
                     const int at = r + tap;
-                    const float x = at < WINDOW ? bf2f(cs[(long long)at * C + c])
-                                                : bf2f(P[(rr.row0 + at - WINDOW) * p_stride + c]);
-                    acc = acc + bf2f(cw[c * TAPS + tap]) * x;
+                    const bf16_t* src = at < WINDOW ? cs + (long long)at * C : P + (rr.row0 + at - WINDOW) * p_stride;
+                    acc = acc + wt[tap] * bf2f(src[c]);
                 }
                 const float act = bfround(acc / (1.0f + expf(-acc)));
                 if (which == 0) qs[i] = act;
                 else if (which == 1) ks[i] = act;
                 else vs[i] = act;
             } else {
-                const int i = t - DK;
-                const float a = bf2f(A[gr * a_stride + h * DK + i]) + dt_bias[h * DK + i];
+                const unsigned i = (unsigned)(t - DK);
+                const float a = bf2f((A + gr * a_stride + h * DK)[i]) + (dt_bias + h * DK)[i];
                 gs[i] = expf(lower * sigmoidf_(decay_rate * a));
             }
         }
         if (t == THREADS - 1) beta_s = bfround(sigmoidf_(bf2f(P[gr * p_stride + b_off + h])));
         __syncthreads();
-        // L2 norms by wave 0: lanes 0..31 take q, lanes 32..63 take k.
         if (wave == 0) {
-            float* x = lane < 32 ? qs : ks;
+            float* x = lane < 32 ? qs : ks;    // lanes 0..31 take q, lanes 32..63 take k
             const int l32 = lane & 31;
             float v4[4];
             const float ss = sumsq128(x, l32, v4);
@@ -122,10 +130,14 @@ __global__ void __launch_bounds__(THREADS) chain_kernel(
             }
         }
         __syncthreads();
-        if (r == 0) {
-#pragma unroll
-            for (int j = 0; j < M::STEPS; ++j) unpack<S>(raw[j], s[j]);
-        }
+    };
+
+    prologue(0);
+
+    int r = 0;
+    do {   // rows >= 1 here; a do-while leaves no zero-trip path that would keep the loaded state alive
+        const long long gr = rr.row0 + r;
+        prologue(r);
         const float beta = beta_s;
         float kk[KPL], qq[KPL], gg[KPL];
 #pragma unroll
@@ -137,19 +149,21 @@ __global__ void __launch_bounds__(THREADS) chain_kernel(
 #pragma unroll
         for (int j = 0; j < M::STEPS; ++j) {
             const int row = M::row(j, wave, lane);
-            update_row<S>(s[j], kk, gg, vs[row], beta);
-            const float o = read_row<S>(s[j], qq);
+            float s[KPL];
+            unpack<S>(raw[j], s);
+            update_row<S>(s, kk, gg, vs[row], beta);
+            const float o = read_row<S>(s, qq);
             if (lane % M::LPR == 0) ys[row] = bfround(o);
+            raw[j] = pack<S>(s);        // rounds a bf16 state (after the row's read-out)
         }
-        round_state<S>(s);
-        if (ckpt != nullptr) store_state<S>(ckpt + (gr * H + h) * (long long)(DV * DK), wave, lane, s);
+        if (ckpt != nullptr) store_raw<S>(ckpt + (gr * H + h) * (long long)(DV * DK), soff_lane, raw);
         if (k_save != nullptr) {
             const long long base = (gr * H + h) * DK;
             if (t < DK) {
-                k_save[base + t] = ks[t];
-                g_save[base + t] = gs[t];
+                (k_save + base)[(unsigned)t] = ks[t];
+                (g_save + base)[(unsigned)t] = gs[t];
             } else {
-                v_save[base + t - DK] = f2bf(vs[t - DK]);
+                (v_save + base)[(unsigned)(t - DK)] = f2bf(vs[t - DK]);
             }
             if (t == 0) b_save[gr * H + h] = beta;
         }
@@ -164,26 +178,18 @@ __global__ void __launch_bounds__(THREADS) chain_kernel(
         if (t < DV) {
             const float yn = ys[t] * rinv_s;
             const float yw = bf2f(norm_w[t]) * yn;
-            const float gate = bf2f(G[gr * g_stride + h * DV + t]);
-            out[gr * out_stride + h * DV + t] = f2bf(yw * sigmoidf_(gate));
+            const float gate = bf2f((G + gr * g_stride + h * DV)[(unsigned)t]);
+            (out + gr * out_stride + h * DV)[(unsigned)t] = f2bf(yw * sigmoidf_(gate));
         }
         __syncthreads();
-    }
-    if (state_out != nullptr) {
-        if (rows == 0) {
-#pragma unroll
-            for (int j = 0; j < M::STEPS; ++j)
-                st128(state_out + sbase + (long long)M::row(j, wave, lane) * DK + key0, raw[j]);
-        } else {
-            store_state<S>(state_out + sbase, wave, lane, s);
-        }
-    }
+    } while (++r < rows);
+    if (state_out != nullptr) store_raw<S>(state_out + sbase, soff_lane, raw);
 }
 
 // Replay of saved rows (reference: kda.cu:214-253, cpu.rs:486-508): workgroup (layer * H + h, b). Waves are
 // independent here: every lane reads its own keys' k and exp(g) and its rows' v straight from the saves.
 template <typename S>
-__global__ void __launch_bounds__(THREADS) replay_kernel(
+__global__ void __launch_bounds__(THREADS, 4) replay_kernel(
         int H, const int32_t* __restrict__ cu_rows, const int32_t* __restrict__ keep, int rows1,
         const S* state_in, S* state_out, long long state_stride, const long long* __restrict__ state_off,
         const float* __restrict__ k_save, const bf16_t* __restrict__ v_save, const float* __restrict__ g_save,
@@ -201,36 +207,32 @@ __global__ void __launch_bounds__(THREADS) replay_kernel(
     const float* gsv = g_save + layer * kv_stride;
     const float* bsv = b_save + layer * b_stride;
     const int key0 = M::key0(lane);
+    const unsigned soff_lane = lane_offset<S>(wave, lane);
+    const unsigned row_lane = (unsigned)M::row(0, wave, lane);
 
     uint4 raw[M::STEPS];
-    load_state<S>(state_in + sbase, wave, lane, raw);
-    if (rows <= 0) {
-#pragma unroll
-        for (int j = 0; j < M::STEPS; ++j)
-            st128(state_out + sbase + (long long)M::row(j, wave, lane) * DK + key0, raw[j]);
-        return;
-    }
-    float s[M::STEPS][KPL];
-#pragma unroll
-    for (int j = 0; j < M::STEPS; ++j) unpack<S>(raw[j], s[j]);
+    load_state<S>(state_in + sbase, soff_lane, raw);
     for (int r = 0; r < rows; ++r) {
         const long long gr = row0 + r;
         const long long base = (gr * H + h) * DK;
         float kk[KPL], gg[KPL];
 #pragma unroll
         for (int c = 0; c < KPL; c += 4) {
-            const float4 k4 = *reinterpret_cast<const float4*>(ksv + base + key0 + c);
-            const float4 g4 = *reinterpret_cast<const float4*>(gsv + base + key0 + c);
+            const float4 k4 = *reinterpret_cast<const float4*>((ksv + base) + (unsigned)(key0 + c));
+            const float4 g4 = *reinterpret_cast<const float4*>((gsv + base) + (unsigned)(key0 + c));
             kk[c] = k4.x; kk[c + 1] = k4.y; kk[c + 2] = k4.z; kk[c + 3] = k4.w;
             gg[c] = g4.x; gg[c + 1] = g4.y; gg[c + 2] = g4.z; gg[c + 3] = g4.w;
         }
         const float beta = bsv[gr * H + h];
 #pragma unroll
-        for (int j = 0; j < M::STEPS; ++j)
-            update_row<S>(s[j], kk, gg, bf2f(vsv[base + M::row(j, wave, lane)]), beta);
-        round_state<S>(s);
+        for (int j = 0; j < M::STEPS; ++j) {
+            float s[KPL];
+            unpack<S>(raw[j], s);
+            update_row<S>(s, kk, gg, bf2f((vsv + base + j * M::RPS)[row_lane]), beta);
+            raw[j] = pack<S>(s);
+        }
     }
-    store_state<S>(state_out + sbase, wave, lane, s);
+    store_raw<S>(state_out + sbase, soff_lane, raw);
 }
 
 // Conv-window shift (reference: kda.cu:258-277, cpu.rs:512-527): lane (channel, layer, request) reads its

@@ -16,11 +16,17 @@ typedef uint16_t bf16_t;
 
 __device__ __forceinline__ float bf2f(bf16_t b) { return __uint_as_float((uint32_t)b << 16); }
 
-// Round to nearest even, NaN quieted: the bits of the reference's bf16::from_f32 (src/bf16.rs:6-13).
-__device__ __forceinline__ bf16_t f2bf(float x) {
-    const uint32_t u = __float_as_uint(x);
-    if (x != x) return (bf16_t)((u >> 16) | 0x0040u);
-    return (bf16_t)((u + (0x7fffu + ((u >> 16) & 1u))) >> 16);
+typedef __bf16 hwbf16x2_t __attribute__((ext_vector_type(2)));
+typedef float hwf32x2_t __attribute__((ext_vector_type(2)));
+
+// Round to nearest even with gfx950's v_cvt_pk_bf16_f32: for every finite or infinite input the bits of the
+// reference's bf16::from_f32 (src/bf16.rs:6-13); a NaN stays a (quiet) NaN.
+__device__ __forceinline__ bf16_t f2bf(float x) { return __builtin_bit_cast(bf16_t, (__bf16)x); }
+
+// Two values in one instruction: lo in bits 0..15, hi in bits 16..31.
+__device__ __forceinline__ uint32_t f2bf2(float lo, float hi) {
+    const hwf32x2_t f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, hwbf16x2_t));
 }
 
 __device__ __forceinline__ float bfround(float x) { return bf2f(f2bf(x)); }
@@ -103,22 +109,45 @@ template <>
 __device__ __forceinline__ uint4 pack<bf16_t>(const float (&s)[8]) {
     uint32_t w[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f2bf(s[2 * i]) | ((uint32_t)f2bf(s[2 * i + 1]) << 16);
+    for (int i = 0; i < 4; ++i) w[i] = f2bf2(s[2 * i], s[2 * i + 1]);
     return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// x[lane ^ M] for M = 1, 2, 4, 8 inside a row of 16 lanes, as data-parallel-primitive moves (no LDS):
+// quad permutes for 1 and 2, a rotation by 8 for 8, and for 4 a shift left into banks 0 and 2 and a shift
+// right into banks 1 and 3 (a bank is 4 lanes).
+template <int M>
+__device__ __forceinline__ float lane_xor16(float x) {
+    const int xi = __float_as_int(x);
+    if constexpr (M == 1) return __int_as_float(__builtin_amdgcn_update_dpp(0, xi, 0xB1, 0xf, 0xf, true));
+    if constexpr (M == 2) return __int_as_float(__builtin_amdgcn_update_dpp(0, xi, 0x4E, 0xf, 0xf, true));
+    if constexpr (M == 8) return __int_as_float(__builtin_amdgcn_update_dpp(0, xi, 0x128, 0xf, 0xf, true));
+    if constexpr (M == 4) {
+        const int lo = __builtin_amdgcn_update_dpp(0, xi, 0x104, 0xf, 0x5, false);     // row_shl:4 -> banks 0, 2
+        return __int_as_float(__builtin_amdgcn_update_dpp(lo, xi, 0x114, 0xf, 0xa, false));  // row_shr:4 -> 1, 3
+    }
+    return x;
 }
 
 // The sum over one value row's 128 keys of per-lane partial sums, in the order of the reference's CPU
 // model (cpu.rs:214-239): partial l (l = 0..31) covers keys 4l..4l+3, then an xor butterfly over l with
 // offsets 16, 8, 4, 2, 1. With NP partials per lane the low bits of l live inside the lane, so the
 // butterfly's first steps cross lanes and its last adds the lane's own partials. Every lane of the row
-// ends with the same bits.
+// ends with the same bits (an addition commutes, so both partners of a step compute the same sum).
 template <int NP, int LPR>
 __device__ __forceinline__ float row_sum(float (&x)[NP]) {
+    if constexpr (LPR == 32) {
 #pragma unroll
-    for (int m = LPR / 2; m >= 1; m >>= 1) {
-#pragma unroll
-        for (int p = 0; p < NP; ++p) x[p] = x[p] + __shfl_xor(x[p], m, 64);
+        for (int p = 0; p < NP; ++p) x[p] = x[p] + __shfl_xor(x[p], 16, 64);
     }
+#pragma unroll
+    for (int p = 0; p < NP; ++p) x[p] = x[p] + lane_xor16<8>(x[p]);
+#pragma unroll
+    for (int p = 0; p < NP; ++p) x[p] = x[p] + lane_xor16<4>(x[p]);
+#pragma unroll
+    for (int p = 0; p < NP; ++p) x[p] = x[p] + lane_xor16<2>(x[p]);
+#pragma unroll
+    for (int p = 0; p < NP; ++p) x[p] = x[p] + lane_xor16<1>(x[p]);
     if (NP == 2) return x[0] + x[1];
     return x[0];
 }
