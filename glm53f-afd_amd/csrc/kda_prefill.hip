@@ -1,24 +1,877 @@
-// Placeholder until the MFMA prefill lands: the entry points exist and refuse to run.
+// KDA chunked prefill on gfx950: the delta rule over a prompt segment in the chunked (WY/UT) form, with every
+// GEMM-shaped step on the matrix cores (v_mfma_f32_16x16x32_{f16,bf16}, f32 accumulation).
+//
+// The algebra is the reference's chunk form (crates/glm53f-kda/src/chunked.rs:67-198; kernel counterpart
+// kda_prefill.cu:95-538 with 16-row chunks on CUDA cores). Here a chunk is 64 rows in four sub-chunks of 16.
+// With G the cumulative log decay inside the chunk, per key channel:
+//   L[i][j] = beta_i sum_d k_i k_j e^{G_i - G_j} (j < i),  M[i][j] = sum_d q_i k_j e^{G_i - G_j} (j <= i),
+//   T = (I + L)^-1,  T' = T diag(beta),  W = T' (k e^G),  U = T' v,  Qg = q e^G,  Kg = k e^{G_last - G};
+//   from the state S entering the chunk: V' = U - W S,  Y = Qg S + M V',  S <- e^{G_last} S + Kg^T V'.
+// e^{G_i - G_j} is factored around a reference row so that both factors are GEMM operands:
+//   * inside a sub-chunk (diagonal 16x16 blocks) around the sub-chunk's first row; one factor reaches e^{+87}
+//     (15 rows at the -5.8 bound), so these operands are bf16 split into hi + lo (three products);
+//   * between sub-chunks around a row in between (the end of a sub-chunk, or the middle of the chunk), where
+//     both exponents are <= 0 and the operands are fp16 (11-bit mantissa at the bf16 MFMA rate).
+// Everything that feeds the state is fp16 or split bf16; T is inverted in f32.
+//
+// Kernels per pass: intra_kernel (one workgroup per chunk, head, request: prologue + L, M, T, W, U, Qg, Kg into
+// the workspace), inter_kernel (one workgroup per head, value-column block, request: the state in MFMA
+// accumulators across the chunks of the pass), then norm_kernel (gated RMSNorm in place) and
+// conv_advance_kernel.
+
 #include "kda_common.h"
 
-extern "C" int64_t glm53f_kda_prefill_workspace_bytes(int32_t, int32_t, int32_t) { return 0; }
-#define UNUSED_PREFILL_ARGS                                                                                       \
-    const glm53f_bf16*, int64_t, int64_t, const glm53f_bf16*, int64_t, const glm53f_bf16*, int64_t
-extern "C" int glm53f_kda_prefill(int32_t, int32_t, UNUSED_PREFILL_ARGS, glm53f_bf16*, const glm53f_bf16*,
-                                  const float*, float*, const float*, const float*, const glm53f_bf16*, float, float,
-                                  glm53f_bf16*, int64_t, int32_t, float*, int64_t, glm53f_stream_t) {
-    return (int)hipErrorNotSupported;
+namespace kda {
+namespace {
+
+constexpr int CH = 64, SUB = 16, THREADS = 256;
+constexpr int NV = 32;                    // value columns per inter workgroup
+constexpr int VBLOCKS = DV / NV;          // inter workgroups per head
+
+typedef _Float16 f16_t;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Workspace of one (request, head, chunk), bytes.
+constexpr int WS_W = 0;                   // fp16 [64 rows][128 keys]
+constexpr int WS_UT = 16384;              // fp16 [128 values][64 rows]
+constexpr int WS_QG = 32768;              // fp16 [64 rows][128 keys]
+constexpr int WS_KGT = 49152;             // fp16 [128 keys][64 rows]
+constexpr int WS_M = 65536;               // fp16 [64 rows][64 rows]
+constexpr int WS_E = 73728;               // f32 [128 keys]: e^{G_last}
+constexpr int WS_BYTES = 74240;
+
+// LDS row strides in 16-bit elements: 128- and 64-wide operand rows padded by 16 bytes, so that the sixteen
+// rows one MFMA fragment read touches fall into distinct banks.
+constexpr int LD128 = 136, LD64 = 72, LDF = 68;   // LDF: f32 [64][68]
+
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float fast_sigmoid(float x) { return fast_rcp(1.0f + fast_exp(-x)); }
+
+__device__ __forceinline__ uint16_t f2h(float x) { return __builtin_bit_cast(uint16_t, (f16_t)x); }
+__device__ __forceinline__ float h2f(uint16_t x) { return (float)__builtin_bit_cast(f16_t, x); }
+
+// One operand fragment of a 16x16x32 MFMA from an LDS array [row][k] (k contiguous): lane l takes row
+// row0 + l % 16, k0 + 8 * (l / 16) .. + 7. The same read serves the A operand (rows = M) and the B operand
+// held transposed (rows = N).
+__device__ __forceinline__ uint4 frag(const uint16_t* base, int ld, int row0, int k0, int lane) {
+    return *reinterpret_cast<const uint4*>(base + (row0 + (lane & 15)) * ld + k0 + 8 * (lane >> 4));
 }
-extern "C" int glm53f_kda_prefill_batch(int32_t, int32_t, const int32_t*, int32_t, UNUSED_PREFILL_ARGS, glm53f_bf16*,
-                                        const int64_t*, const glm53f_bf16*, const float*, float*, const int64_t*,
-                                        const float*, const float*, const glm53f_bf16*, float, float, glm53f_bf16*,
-                                        int64_t, int32_t, float*, int64_t, glm53f_stream_t) {
-    return (int)hipErrorNotSupported;
+
+__device__ __forceinline__ f32x4 mfma_f16(uint4 a, uint4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
-extern "C" int glm53f_kda_prefill_batch_bf16state(int32_t, int32_t, const int32_t*, int32_t, UNUSED_PREFILL_ARGS,
-                                                  glm53f_bf16*, const int64_t*, const glm53f_bf16*,
-                                                  const glm53f_bf16*, glm53f_bf16*, const int64_t*, const float*,
-                                                  const float*, const glm53f_bf16*, float, float, glm53f_bf16*,
-                                                  int64_t, int32_t, float*, int64_t, glm53f_stream_t) {
-    return (int)hipErrorNotSupported;
+__device__ __forceinline__ f32x4 mfma_bf16(uint4 a, uint4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0,
+                                                   0);
+}
+
+// C[16][16] += A[a_row0 ..][0, K) . B^T[b_row0 ..][0, K) with fp16 operands.
+__device__ __forceinline__ f32x4 tile_f16(const uint16_t* a, int a_row0, int lda, const uint16_t* b, int b_row0, int ldb,
+                                          int K, int lane, f32x4 acc) {
+    for (int k0 = 0; k0 < K; k0 += 32) acc = mfma_f16(frag(a, lda, a_row0, k0, lane), frag(b, ldb, b_row0, k0, lane), acc);
+    return acc;
+}
+
+// The same with bf16 operands split into hi + lo: a_hi b_hi + a_hi b_lo + a_lo b_hi.
+__device__ __forceinline__ f32x4 tile_bf16x3(const uint16_t* ah, const uint16_t* al, int a_row0, const uint16_t* bh,
+                                             const uint16_t* bl, int b_row0, int lane, f32x4 acc) {
+    for (int k0 = 0; k0 < DK; k0 += 32) {
+        const uint4 fah = frag(ah, LD128, a_row0, k0, lane), fal = frag(al, LD128, a_row0, k0, lane);
+        const uint4 fbh = frag(bh, LD128, b_row0, k0, lane), fbl = frag(bl, LD128, b_row0, k0, lane);
+        acc = mfma_bf16(fal, fbh, acc);
+        acc = mfma_bf16(fah, fbl, acc);
+        acc = mfma_bf16(fah, fbh, acc);
+    }
+    return acc;
+}
+
+// bf16 hi + lo of x: hi = bf16(x), lo = bf16(x - hi).
+__device__ __forceinline__ void split_bf16(float x, uint16_t& hi, uint16_t& lo) {
+    hi = f2bf(x);
+    lo = f2bf(x - bf2f(hi));
+}
+
+// LDS map of intra_kernel, bytes.
+constexpr int I_TOT = 0;                          // f32 [4][128]: log-decay totals of the sub-chunks
+constexpr int I_BETA = I_TOT + 4 * DK * 4;        // f32 [64]
+constexpr int I_INV = I_BETA + CH * 4;            // f32 [2][64]: 1/|q| * 128^-0.5, 1/|k|
+constexpr int I_KET = I_INV + 2 * CH * 4;         // fp16 [128 keys][LD64]: k e^G, transposed
+constexpr int I_VT = I_KET + DK * LD64 * 2;       // fp16 [128 values][LD64]: v, transposed
+constexpr int I_L = I_VT + DV * LD64 * 2;         // f32 [64][LDF]: L
+constexpr int I_KC1 = I_L + CH * LDF * 4;         // fp16 [32][LD128]: column side around the chunk's middle
+constexpr int I_PASS = I_KC1 + 32 * LD128 * 2;    // the rest is reused by every half
+constexpr int P_ROWS32 = 32 * LD128 * 2;          // one [32][LD128] 16-bit array
+constexpr int P_ROWS16 = 16 * LD128 * 2;
+constexpr int I_DIAG = I_PASS;                    // six [32][LD128] bf16 arrays: KrD hi/lo, QrD hi/lo, KcD hi/lo
+constexpr int I_RAWQ = I_PASS;                    // raw q, k (bf16) before the norms: dead before the operands land
+constexpr int I_RAWK = I_PASS + P_ROWS32;
+constexpr int I_R2 = I_DIAG + 6 * P_ROWS32;       // KR2, QR2, KC2: three [16][LD128] fp16 arrays
+constexpr int I_R1 = I_R2 + 3 * P_ROWS16;         // KR1, QR1: two [32][LD128] fp16 arrays
+constexpr int I_END = I_R1 + 2 * P_ROWS32;
+// After the halves: the inverse.
+constexpr int I_T = I_PASS;                       // f32 [64][LDF]
+constexpr int I_X = I_T + CH * LDF * 4;           // f32 [64][LDF]
+constexpr int I_TQ = I_X + CH * LDF * 4;          // fp16 [64][LD64]: T diag(beta)
+constexpr int INTRA_LDS = I_END;
+static_assert(I_TQ + CH * LD64 * 2 <= I_END, "inverse scratch must fit the per-half region");
+static_assert(INTRA_LDS <= 160 * 1024, "intra_kernel LDS");
+
+// Pass 1: one chunk of one head of one request, everything that does not need the state, into its workspace slot.
+__global__ void __launch_bounds__(THREADS) intra_kernel(
+        int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
+        const bf16_t* __restrict__ P, long long p_stride, long long b_off, const bf16_t* __restrict__ A,
+        long long a_stride, const bf16_t* __restrict__ conv, const long long* __restrict__ conv_off,
+        const bf16_t* __restrict__ cw, const float* __restrict__ a_log, const float* __restrict__ dt_bias, float lower,
+        unsigned char* __restrict__ ws) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const RowRange rr = request_rows(cu_rows, b, rows1);
+    const int r0 = sub0 + c * CH;                 // the chunk's first row inside the request
+    const int n = min(CH, rr.rows - r0);          // its real rows
+    if (n <= 0) return;
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+    const int d = t & (DK - 1), s = t >> 7;       // this lane's channel, and which sub-chunk of a half it takes
+    const long long C = 3LL * H * DK;
+    const bf16_t* cs = conv + (conv_off != nullptr ? conv_off[b] : 0);
+    unsigned char* wsc = ws + (((long long)b * H + h) * chunks + c) * (long long)WS_BYTES;
+
+    float* tot = reinterpret_cast<float*>(smem + I_TOT);
+    float* beta_s = reinterpret_cast<float*>(smem + I_BETA);
+    float* inv_s = reinterpret_cast<float*>(smem + I_INV);
+    uint16_t* keT = reinterpret_cast<uint16_t*>(smem + I_KET);
+    uint16_t* VT = reinterpret_cast<uint16_t*>(smem + I_VT);
+    float* Ls = reinterpret_cast<float*>(smem + I_L);
+    uint16_t* KC1 = reinterpret_cast<uint16_t*>(smem + I_KC1);
+
+    // ---- gates of the whole chunk: cumulative log decay of this lane's channel inside its two sub-chunks
+    const float rate = fast_exp(a_log[h]);
+    const float dtb = dt_bias[h * DK + d];
+    float cg[2][SUB];                             // inclusive cumulative sums, sub-chunks s and 2 + s
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+        const int a = 2 * h2 + s;
+        float run = 0.0f;
+#pragma unroll
+        for (int i = 0; i < SUB; ++i) {
+            const int R = SUB * a + i;
+            float g = 0.0f;
+            if (R < n) {
+                const float av = bf2f((A + (rr.row0 + r0 + R) * a_stride + h * DK)[(unsigned)d]);
+                g = lower * fast_sigmoid(rate * (av + dtb));
+            }
+            run += g;
+            cg[h2][i] = run;
+        }
+        tot[a * DK + d] = run;
+    }
+    if (t < CH) {
+        float bv = 0.0f;
+        if (t < n) bv = bfround(fast_sigmoid(bf2f(P[(rr.row0 + r0 + t) * p_stride + b_off + h])));
+        beta_s[t] = bv;
+    }
+    // conv weights of this lane's q, k and v channels
+    const unsigned cq = (unsigned)(h * DK + d), ck = (unsigned)(H * DK + h * DK + d), cv = (unsigned)(2 * H * DK + h * DK + d);
+    float wq[TAPS], wk[TAPS], wv[TAPS];
+    {
+        const uint2 a4 = *reinterpret_cast<const uint2*>(cw + (size_t)cq * TAPS);
+        const uint2 b4 = *reinterpret_cast<const uint2*>(cw + (size_t)ck * TAPS);
+        const uint2 c4 = *reinterpret_cast<const uint2*>(cw + (size_t)cv * TAPS);
+        wq[0] = __uint_as_float(a4.x << 16); wq[1] = __uint_as_float(a4.x & 0xffff0000u);
+        wq[2] = __uint_as_float(a4.y << 16); wq[3] = __uint_as_float(a4.y & 0xffff0000u);
+        wk[0] = __uint_as_float(b4.x << 16); wk[1] = __uint_as_float(b4.x & 0xffff0000u);
+        wk[2] = __uint_as_float(b4.y << 16); wk[3] = __uint_as_float(b4.y & 0xffff0000u);
+        wv[0] = __uint_as_float(c4.x << 16); wv[1] = __uint_as_float(c4.x & 0xffff0000u);
+        wv[2] = __uint_as_float(c4.y << 16); wv[3] = __uint_as_float(c4.y & 0xffff0000u);
+    }
+    __syncthreads();
+    // prefix and suffix totals of this lane's channel: B[a] = sum of tot over sub-chunks before a
+    float Bp[5];
+    Bp[0] = 0.0f;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) Bp[a + 1] = Bp[a] + tot[a * DK + d];
+    if (s == 0) reinterpret_cast<float*>(wsc + WS_E)[d] = fast_exp(Bp[4]);
+
+    // Row `rel` (relative to the request's first row; -3..-1 are the conv window) of channel ch, 0 past the end.
+    auto input = [&](int rel, unsigned ch) -> float {
+        if (rel >= rr.rows) return 0.0f;
+        const bf16_t* src = rel < 0 ? cs + (long long)(rel + WINDOW) * C : P + (rr.row0 + rel) * p_stride;
+        return bf2f(src[ch]);
+    };
+
+    // ---- the two halves of the chunk: sub-chunks {0, 1}, then {2, 3}
+#pragma unroll 1
+    for (int h2 = 0; h2 < 2; ++h2) {
+        const int a = 2 * h2 + s;                 // this lane's sub-chunk
+        const int lr0 = SUB * s;                  // its first row inside the half's 32-row arrays
+        uint16_t* rawq = reinterpret_cast<uint16_t*>(smem + I_RAWQ);
+        uint16_t* rawk = reinterpret_cast<uint16_t*>(smem + I_RAWK);
+        // conv + SiLU, one bf16 rounding, 16 rows of q, k, v
+        float qr[SUB], kr[SUB];
+        {
+            const int rel0 = r0 + SUB * a;
+            float xq[TAPS], xk[TAPS], xv[TAPS];
+#pragma unroll
+            for (int j = 0; j < WINDOW; ++j) {
+                xq[j + 1] = input(rel0 - WINDOW + j, cq);
+                xk[j + 1] = input(rel0 - WINDOW + j, ck);
+                xv[j + 1] = input(rel0 - WINDOW + j, cv);
+            }
+            uint32_t vpack[SUB / 2];
+#pragma unroll
+            for (int i = 0; i < SUB; ++i) {
+#pragma unroll
+                for (int j = 0; j < WINDOW; ++j) { xq[j] = xq[j + 1]; xk[j] = xk[j + 1]; xv[j] = xv[j + 1]; }
+                const bool live = SUB * a + i < n;
+                xq[3] = live ? input(rel0 + i, cq) : 0.0f;
+                xk[3] = live ? input(rel0 + i, ck) : 0.0f;
+                xv[3] = live ? input(rel0 + i, cv) : 0.0f;
+                float aq = 0.0f, ak = 0.0f, av = 0.0f;
+#pragma unroll
+                for (int tap = 0; tap < TAPS; ++tap) {
+                    aq = __builtin_fmaf(wq[tap], xq[tap], aq);
+                    ak = __builtin_fmaf(wk[tap], xk[tap], ak);
+                    av = __builtin_fmaf(wv[tap], xv[tap], av);
+                }
+                const float sq = live ? bfround(aq * fast_sigmoid(aq)) : 0.0f;
+                const float sk = live ? bfround(ak * fast_sigmoid(ak)) : 0.0f;
+                const float sv = live ? bfround(av * fast_sigmoid(av)) : 0.0f;
+                qr[i] = sq;
+                kr[i] = sk;
+                rawq[(lr0 + i) * LD128 + d] = f2bf(sq);
+                rawk[(lr0 + i) * LD128 + d] = f2bf(sk);
+                const uint32_t hv = f2h(sv);        // a bf16 value is exact in fp16 (but for values below 2^-14)
+                if (i & 1) vpack[i / 2] |= hv << 16; else vpack[i / 2] = hv;
+            }
+            uint4* dst = reinterpret_cast<uint4*>(VT + d * LD64 + SUB * a);
+            dst[0] = make_uint4(vpack[0], vpack[1], vpack[2], vpack[3]);
+            dst[1] = make_uint4(vpack[4], vpack[5], vpack[6], vpack[7]);
+        }
+        __syncthreads();
+        // L2 norms of the half's 32 rows of q and k: four lanes per (row, q|k), 32 channels each
+        {
+            const int task = t >> 2, part = t & 3;
+            const int row = task & 31, which = task >> 5;
+            const uint16_t* src = (which == 0 ? rawq : rawk) + row * LD128 + 32 * part;
+            float ss = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint4 u = *reinterpret_cast<const uint4*>(src + 8 * j);
+                const uint32_t wds[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float lo = __uint_as_float(wds[e] << 16), hi = __uint_as_float(wds[e] & 0xffff0000u);
+                    ss = __builtin_fmaf(lo, lo, ss);
+                    ss = __builtin_fmaf(hi, hi, ss);
+                }
+            }
+            ss = ss + lane_xor16<1>(ss);
+            ss = ss + lane_xor16<2>(ss);
+            if (part == 0) {
+                float inv = __builtin_amdgcn_rsqf(ss + 1e-6f);
+                if (which == 0) inv *= 0.08838834764831845f;   // 128^-0.5
+                inv_s[which * CH + 32 * h2 + row] = inv;
+            }
+        }
+        __syncthreads();
+        // operands of this lane's 16 rows
+        {
+            uint16_t* KrDh = reinterpret_cast<uint16_t*>(smem + I_DIAG);
+            uint16_t* KrDl = KrDh + 32 * LD128;
+            uint16_t* QrDh = KrDl + 32 * LD128;
+            uint16_t* QrDl = QrDh + 32 * LD128;
+            uint16_t* KcDh = QrDl + 32 * LD128;
+            uint16_t* KcDl = KcDh + 32 * LD128;
+            uint16_t* KR2 = reinterpret_cast<uint16_t*>(smem + I_R2);
+            uint16_t* QR2 = KR2 + 16 * LD128;
+            uint16_t* KC2 = QR2 + 16 * LD128;
+            uint16_t* KR1 = reinterpret_cast<uint16_t*>(smem + I_R1);
+            uint16_t* QR1 = KR1 + 32 * LD128;
+            const float g0 = cg[h2][0];
+            const float eneg0 = fast_exp(-g0);                 // e^{-g of the sub-chunk's first row}
+            const float ep_last = fast_exp(cg[h2][SUB - 1] - g0);
+            const float eB = fast_exp(Bp[a]);                   // e^{G before this sub-chunk}
+            const float eSuf = fast_exp(Bp[4] - Bp[a + 1]);     // e^{G_last - G at this sub-chunk's end}
+            // around the chunk's middle: columns of sub-chunk 0 still cross sub-chunk 1, rows of 3 crossed 2
+            const float eMid = (a == 0) ? fast_exp(tot[1 * DK + d]) : (a == 3 ? fast_exp(tot[2 * DK + d]) : 1.0f);
+            uint32_t kepack[SUB / 2], kgpack[SUB / 2];
+#pragma unroll
+            for (int i = 0; i < SUB; ++i) {
+                const int R = SUB * a + i;
+                const float kh = kr[i] * inv_s[CH + R], qh = qr[i] * inv_s[R];
+                const float e1 = fast_exp(cg[h2][i]);           // e^{G_i - G at the sub-chunk's start}
+                const float ep = e1 * eneg0;                    // e^{G_i - G_first}
+                const float rp = fast_rcp(ep);                  // e^{G_first - G_i}, up to e^87
+                const float col2 = ep_last * rp;                // e^{G at the sub-chunk's end - G_i}
+                const int lr = lr0 + i;
+                uint16_t hi, lo;
+                split_bf16(kh * ep, hi, lo); KrDh[lr * LD128 + d] = hi; KrDl[lr * LD128 + d] = lo;
+                split_bf16(qh * ep, hi, lo); QrDh[lr * LD128 + d] = hi; QrDl[lr * LD128 + d] = lo;
+                split_bf16(kh * rp, hi, lo); KcDh[lr * LD128 + d] = hi; KcDl[lr * LD128 + d] = lo;
+                if (s == 1) {
+                    KR2[i * LD128 + d] = f2h(kh * e1);
+                    QR2[i * LD128 + d] = f2h(qh * e1);
+                } else {
+                    KC2[i * LD128 + d] = f2h(kh * col2);
+                }
+                if (h2 == 0) {
+                    KC1[lr * LD128 + d] = f2h(kh * col2 * eMid);
+                } else {
+                    KR1[lr * LD128 + d] = f2h(kh * e1 * eMid);
+                    QR1[lr * LD128 + d] = f2h(qh * e1 * eMid);
+                }
+                const uint32_t ke = f2h(kh * e1 * eB), kg = f2h(kh * col2 * eSuf);
+                if (i & 1) { kepack[i / 2] |= ke << 16; kgpack[i / 2] |= kg << 16; }
+                else { kepack[i / 2] = ke; kgpack[i / 2] = kg; }
+                reinterpret_cast<uint16_t*>(wsc + WS_QG)[R * DK + d] = f2h(qh * e1 * eB);
+            }
+            uint4* kd = reinterpret_cast<uint4*>(keT + d * LD64 + SUB * a);
+            kd[0] = make_uint4(kepack[0], kepack[1], kepack[2], kepack[3]);
+            kd[1] = make_uint4(kepack[4], kepack[5], kepack[6], kepack[7]);
+            uint4* gd = reinterpret_cast<uint4*>(wsc + WS_KGT + (d * CH + SUB * a) * 2);
+            gd[0] = make_uint4(kgpack[0], kgpack[1], kgpack[2], kgpack[3]);
+            gd[1] = make_uint4(kgpack[4], kgpack[5], kgpack[6], kgpack[7]);
+        }
+        __syncthreads();
+        // the half's blocks of L and M on the matrix cores
+        {
+            const uint16_t* KrDh = reinterpret_cast<const uint16_t*>(smem + I_DIAG);
+            const uint16_t* KrDl = KrDh + 32 * LD128;
+            const uint16_t* QrDh = KrDl + 32 * LD128;
+            const uint16_t* QrDl = QrDh + 32 * LD128;
+            const uint16_t* KcDh = QrDl + 32 * LD128;
+            const uint16_t* KcDl = KcDh + 32 * LD128;
+            const uint16_t* KR2 = reinterpret_cast<const uint16_t*>(smem + I_R2);
+            const uint16_t* QR2 = KR2 + 16 * LD128;
+            const uint16_t* KC2 = QR2 + 16 * LD128;
+            const uint16_t* KR1 = reinterpret_cast<const uint16_t*>(smem + I_R1);
+            const uint16_t* QR1 = KR1 + 32 * LD128;
+            uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
+            const int rl = 4 * (lane >> 4), cl = lane & 15;   // this lane's rows rl..rl+3 and column cl of a tile
+            // Store a finished tile at block (rb, cb): L = beta_i * acc (strictly lower on the diagonal) to LDS,
+            // M (lower with the diagonal) to the workspace.
+            auto put_L = [&](f32x4 acc, int rb, int cb) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int gi = SUB * rb + rl + r, gj = SUB * cb + cl;
+                    Ls[gi * LDF + gj] = (rb != cb || gj < gi) ? beta_s[gi] * acc[r] : 0.0f;
+                }
+            };
+            auto put_M = [&](f32x4 acc, int rb, int cb) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int gi = SUB * rb + rl + r, gj = SUB * cb + cl;
+                    Mg[gi * CH + gj] = f2h((rb != cb || gj <= gi) ? acc[r] : 0.0f);
+                }
+            };
+            const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+            // diagonal blocks: waves 0, 1 take L of sub-chunks 2 h2, 2 h2 + 1; waves 2, 3 take M
+            {
+                const int sub = wave & 1, blk = 2 * h2 + sub;
+                if (wave < 2) put_L(tile_bf16x3(KrDh, KrDl, SUB * sub, KcDh, KcDl, SUB * sub, lane, zero), blk, blk);
+                else put_M(tile_bf16x3(QrDh, QrDl, SUB * sub, KcDh, KcDl, SUB * sub, lane, zero), blk, blk);
+            }
+            // the block between the half's two sub-chunks
+            if (wave == 0) put_L(tile_f16(KR2, 0, LD128, KC2, 0, LD128, DK, lane, zero), 2 * h2 + 1, 2 * h2);
+            if (wave == 2) put_M(tile_f16(QR2, 0, LD128, KC2, 0, LD128, DK, lane, zero), 2 * h2 + 1, 2 * h2);
+            // rows of the second half against columns of the first
+            if (h2 == 1) {
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const int idx = 2 * wave + q;              // 0..3: L tiles, 4..7: M tiles
+                    const int ra = (idx >> 1) & 1, cb = idx & 1;
+                    if (idx < 4) put_L(tile_f16(KR1, SUB * ra, LD128, KC1, SUB * cb, LD128, DK, lane, zero), 2 + ra, cb);
+                    else put_M(tile_f16(QR1, SUB * ra, LD128, KC1, SUB * cb, LD128, DK, lane, zero), 2 + ra, cb);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    // M above the block diagonal is zero: blocks (0,1), (0,2), (0,3), (1,2), (1,3), (2,3)
+    {
+        uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
+        for (int e = t; e < 6 * 256; e += THREADS) {
+            const int blk = e >> 8, r = (e >> 4) & 15, cc = e & 15;
+            const int rb = blk < 3 ? 0 : (blk < 5 ? 1 : 2);
+            const int cb = blk < 3 ? blk + 1 : (blk < 5 ? blk - 1 : 3);
+            Mg[(SUB * rb + r) * CH + SUB * cb + cc] = 0;
+        }
+    }
+
+    // ---- T = (I + L)^-1 in f32
+    float* Ts = reinterpret_cast<float*>(smem + I_T);
+    float* Xs = reinterpret_cast<float*>(smem + I_X);
+    uint16_t* Tq = reinterpret_cast<uint16_t*>(smem + I_TQ);
+    if (t < CH) {
+        // diagonal blocks by forward substitution: lane (a, j) solves column j of block a
+        const int a = t >> 4, j = t & 15;
+        float x[SUB];
+#pragma unroll
+        for (int i = 0; i < SUB; ++i) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int m = 0; m < i; ++m) acc = __builtin_fmaf(Ls[(SUB * a + i) * LDF + SUB * a + m], x[m], acc);
+            x[i] = i < j ? 0.0f : (i == j ? 1.0f : -acc);
+            Ts[(SUB * a + i) * LDF + SUB * a + j] = x[i];
+        }
+    }
+    __syncthreads();
+    // off-diagonal blocks by distance from the diagonal: T_ab = -T_aa sum_{c=b}^{a-1} L_ac T_cb
+    {
+        const int ei = t >> 4, ej = t & 15;       // this lane's element of a 16x16 block
+#pragma unroll 1
+        for (int dist = 1; dist < 4; ++dist) {
+            for (int bb = 0; bb + dist < 4; ++bb) {
+                const int a = bb + dist;
+                float acc = 0.0f;
+                for (int cc = bb; cc < a; ++cc)
+#pragma unroll
+                    for (int m = 0; m < SUB; ++m)
+                        acc = __builtin_fmaf(Ls[(SUB * a + ei) * LDF + SUB * cc + m], Ts[(SUB * cc + m) * LDF + SUB * bb + ej], acc);
+                Xs[(SUB * a + ei) * LDF + SUB * bb + ej] = acc;
+            }
+            __syncthreads();
+            for (int bb = 0; bb + dist < 4; ++bb) {
+                const int a = bb + dist;
+                float acc = 0.0f;
+#pragma unroll
+                for (int m = 0; m < SUB; ++m)
+                    acc = __builtin_fmaf(Ts[(SUB * a + ei) * LDF + SUB * a + m], Xs[(SUB * a + m) * LDF + SUB * bb + ej], acc);
+                Ts[(SUB * a + ei) * LDF + SUB * bb + ej] = -acc;
+            }
+            __syncthreads();
+        }
+    }
+    // T' = T diag(beta) as an fp16 operand (zero above the diagonal)
+    for (int e = t; e < CH * CH; e += THREADS) {
+        const int i = e >> 6, j = e & 63;
+        Tq[i * LD64 + j] = f2h((j >> 4) <= (i >> 4) ? Ts[i * LDF + j] * beta_s[j] : 0.0f);
+    }
+    __syncthreads();
+
+    // ---- W = T' (k e^G) and U = T' v
+    {
+        const int rl = 4 * (lane >> 4), cl = lane & 15;
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        // W transposed: tile [16 keys][16 rows], so a lane ends with four consecutive keys of one row
+#pragma unroll
+        for (int mt = 2 * wave; mt < 2 * wave + 2; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) {
+                const f32x4 acc = tile_f16(keT, SUB * mt, LD64, Tq, SUB * nt, LD64, CH, lane, zero);
+                const uint32_t w0 = (uint32_t)f2h(acc[0]) | ((uint32_t)f2h(acc[1]) << 16);
+                const uint32_t w1 = (uint32_t)f2h(acc[2]) | ((uint32_t)f2h(acc[3]) << 16);
+                *reinterpret_cast<uint2*>(wsc + WS_W + ((SUB * nt + cl) * DK + SUB * mt + rl) * 2) = make_uint2(w0, w1);
+            }
+        // U: tile [16 rows][16 values], stored transposed: four consecutive rows of one value column
+#pragma unroll
+        for (int nt = 2 * wave; nt < 2 * wave + 2; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt) {
+                const f32x4 acc = tile_f16(Tq, SUB * mt, LD64, VT, SUB * nt, LD64, CH, lane, zero);
+                const uint32_t u0 = (uint32_t)f2h(acc[0]) | ((uint32_t)f2h(acc[1]) << 16);
+                const uint32_t u1 = (uint32_t)f2h(acc[2]) | ((uint32_t)f2h(acc[3]) << 16);
+                *reinterpret_cast<uint2*>(wsc + WS_UT + ((SUB * nt + cl) * CH + SUB * mt + rl) * 2) = make_uint2(u0, u1);
+            }
+    }
+}
+
+// LDS map of inter_kernel, bytes.
+constexpr int N_W = 0;                            // fp16 [64][LD128]
+constexpr int N_Q = N_W + CH * LD128 * 2;         // fp16 [64][LD128]
+constexpr int N_K = N_Q + CH * LD128 * 2;         // fp16 [128][LD64]: Kg transposed
+constexpr int N_M = N_K + DK * LD64 * 2;          // fp16 [64][LD64]
+constexpr int N_U = N_M + CH * LD64 * 2;          // fp16 [NV][LD64]: this block's columns of U, transposed
+constexpr int N_E = N_U + NV * LD64 * 2;          // f32 [128]
+constexpr int N_S = N_E + DK * 4;                 // fp16 [NV][LD128]: the state, transposed
+constexpr int N_V = N_S + NV * LD128 * 2;         // fp16 [NV][LD64]: V', transposed
+constexpr int INTER_LDS = N_V + NV * LD64 * 2;
+static_assert(INTER_LDS <= 160 * 1024, "inter_kernel LDS");
+// 16-byte pieces of one chunk's workspace a workgroup stages: W, Qg, Kg^T, M, its slice of U^T, e^{G_last}.
+constexpr int STAGE_VEC = (16384 + 16384 + 16384 + 8192 + NV * CH * 2 + 512) / 16;
+constexpr int STAGE_PER_LANE = (STAGE_VEC + THREADS - 1) / THREADS;
+
+template <typename S>
+__device__ __forceinline__ float load_state_elem4(const S* p, float (&v)[4]);
+template <>
+__device__ __forceinline__ float load_state_elem4<float>(const float* p, float (&v)[4]) {
+    const float4 x = *reinterpret_cast<const float4*>(p);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+    return 0.0f;
+}
+template <>
+__device__ __forceinline__ float load_state_elem4<bf16_t>(const bf16_t* p, float (&v)[4]) {
+    const uint2 x = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(x.x << 16); v[1] = __uint_as_float(x.x & 0xffff0000u);
+    v[2] = __uint_as_float(x.y << 16); v[3] = __uint_as_float(x.y & 0xffff0000u);
+    return 0.0f;
+}
+__device__ __forceinline__ void store_state_elem4(float* p, const f32x4 v) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store_state_elem4(bf16_t* p, const f32x4 v) {
+    *reinterpret_cast<uint2*>(p) = make_uint2(f2bf2(v[0], v[1]), f2bf2(v[2], v[3]));
+}
+
+// Pass 2: one head's NV value columns of one request through the chunks of the pass, in order. The state
+// S[128 keys][NV] lives in MFMA accumulators: wave w owns keys 32 w .. 32 w + 31.
+template <typename S>
+__global__ void __launch_bounds__(THREADS) inter_kernel(
+        int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
+        const S* state_in, S* state_out, const long long* __restrict__ state_off,
+        bf16_t* __restrict__ out, long long out_stride, const unsigned char* __restrict__ ws) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int h = blockIdx.x / VBLOCKS, vb = blockIdx.x % VBLOCKS, b = blockIdx.y;
+    const RowRange rr = request_rows(cu_rows, b, rows1);
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+    const int left = rr.rows - sub0;                              // rows of this request from this pass on
+    const int nch = left <= 0 ? 0 : min(chunks, (left + CH - 1) / CH);
+    if (nch == 0 && sub0 > 0) return;                             // nothing left: the state is already written
+    const long long sbase = (state_off != nullptr ? state_off[b] : 0) + (long long)h * DV * DK;
+    const int rl = 4 * (lane >> 4), cl = lane & 15;
+
+    uint16_t* Wl = reinterpret_cast<uint16_t*>(smem + N_W);
+    uint16_t* Ql = reinterpret_cast<uint16_t*>(smem + N_Q);
+    uint16_t* Kl = reinterpret_cast<uint16_t*>(smem + N_K);
+    uint16_t* Ml = reinterpret_cast<uint16_t*>(smem + N_M);
+    uint16_t* Ul = reinterpret_cast<uint16_t*>(smem + N_U);
+    float* El = reinterpret_cast<float*>(smem + N_E);
+    uint16_t* Sl = reinterpret_cast<uint16_t*>(smem + N_S);
+    uint16_t* Vl = reinterpret_cast<uint16_t*>(smem + N_V);
+
+    // the state: accS[mt][nt][r] = S[key 32 w + 16 mt + rl + r][value NV vb + 16 nt + cl]
+    f32x4 accS[2][2];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            float v4[4];
+            load_state_elem4<S>(state_in + sbase + (long long)(NV * vb + SUB * nt + cl) * DK + 32 * wave + SUB * mt + rl, v4);
+            accS[mt][nt] = f32x4{v4[0], v4[1], v4[2], v4[3]};
+        }
+
+    const unsigned char* wsh = ws + ((long long)b * H + h) * chunks * (long long)WS_BYTES;
+    // Staging of a chunk's workspace: global -> registers (issued a chunk ahead) -> LDS.
+    uint4 stage[STAGE_PER_LANE];
+    auto stage_load = [&](int c) {
+        const unsigned char* src = wsh + (long long)c * WS_BYTES;
+#pragma unroll
+        for (int q = 0; q < STAGE_PER_LANE; ++q) {
+            const int v = q * THREADS + t;
+            if (v < STAGE_VEC) {
+                int off;   // piece index -> byte offset in the workspace
+                if (v < 1024) off = WS_W + v * 16;
+                else if (v < 2048) off = WS_QG + (v - 1024) * 16;
+                else if (v < 3072) off = WS_KGT + (v - 2048) * 16;
+                else if (v < 3584) off = WS_M + (v - 3072) * 16;
+                else if (v < 3584 + NV * CH / 8) off = WS_UT + NV * vb * CH * 2 + (v - 3584) * 16;
+                else off = WS_E + (v - 3584 - NV * CH / 8) * 16;
+                stage[q] = *reinterpret_cast<const uint4*>(src + off);
+            }
+        }
+    };
+    auto stage_store = [&]() {
+#pragma unroll
+        for (int q = 0; q < STAGE_PER_LANE; ++q) {
+            const int v = q * THREADS + t;
+            if (v < STAGE_VEC) {
+                unsigned char* dst;
+                if (v < 1024) dst = smem + N_W + ((v >> 4) * LD128 + (v & 15) * 8) * 2;                 // 16 pieces per row
+                else if (v < 2048) dst = smem + N_Q + (((v - 1024) >> 4) * LD128 + ((v - 1024) & 15) * 8) * 2;
+                else if (v < 3072) dst = smem + N_K + (((v - 2048) >> 3) * LD64 + ((v - 2048) & 7) * 8) * 2;  // 8 per row
+                else if (v < 3584) dst = smem + N_M + (((v - 3072) >> 3) * LD64 + ((v - 3072) & 7) * 8) * 2;
+                else if (v < 3584 + NV * CH / 8) dst = smem + N_U + (((v - 3584) >> 3) * LD64 + ((v - 3584) & 7) * 8) * 2;
+                else dst = smem + N_E + (v - 3584 - NV * CH / 8) * 16;
+                *reinterpret_cast<uint4*>(dst) = stage[q];
+            }
+        }
+    };
+    // S^T for the first chunk
+    auto put_state = [&]() {
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) {
+                const uint32_t s0 = (uint32_t)f2h(accS[mt][nt][0]) | ((uint32_t)f2h(accS[mt][nt][1]) << 16);
+                const uint32_t s1 = (uint32_t)f2h(accS[mt][nt][2]) | ((uint32_t)f2h(accS[mt][nt][3]) << 16);
+                *reinterpret_cast<uint2*>(Sl + (SUB * nt + cl) * LD128 + 32 * wave + SUB * mt + rl) = make_uint2(s0, s1);
+            }
+    };
+
+    if (nch > 0) stage_load(0);
+    for (int c = 0; c < nch; ++c) {
+        const int nrows = min(CH, left - c * CH);
+        stage_store();
+        put_state();
+        __syncthreads();
+        if (c + 1 < nch) stage_load(c + 1);
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        // V' = U - W S: wave w takes rows 16 w .. 16 w + 15
+        uint4 sfrag[2][4];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) sfrag[nt][ks] = frag(Sl, LD128, SUB * nt, 32 * ks, lane);
+        f32x4 accV[2] = {zero, zero};
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const uint4 a = frag(Wl, LD128, SUB * wave, 32 * ks, lane);
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) accV[nt] = mfma_f16(a, sfrag[nt][ks], accV[nt]);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            const uint2 u = *reinterpret_cast<const uint2*>(Ul + (SUB * nt + cl) * LD64 + SUB * wave + rl);
+            const float v0 = h2f((uint16_t)(u.x & 0xffffu)) - accV[nt][0], v1 = h2f((uint16_t)(u.x >> 16)) - accV[nt][1];
+            const float v2 = h2f((uint16_t)(u.y & 0xffffu)) - accV[nt][2], v3 = h2f((uint16_t)(u.y >> 16)) - accV[nt][3];
+            const uint32_t p0 = (uint32_t)f2h(v0) | ((uint32_t)f2h(v1) << 16);
+            const uint32_t p1 = (uint32_t)f2h(v2) | ((uint32_t)f2h(v3) << 16);
+            *reinterpret_cast<uint2*>(Vl + (SUB * nt + cl) * LD64 + SUB * wave + rl) = make_uint2(p0, p1);
+        }
+        __syncthreads();
+        // Y = Qg S + M V'
+        uint4 vfrag[2][2];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) vfrag[nt][ks] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
+        f32x4 accY[2] = {zero, zero};
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const uint4 a = frag(Ql, LD128, SUB * wave, 32 * ks, lane);
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) accY[nt] = mfma_f16(a, sfrag[nt][ks], accY[nt]);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const uint4 a = frag(Ml, LD64, SUB * wave, 32 * ks, lane);
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) accY[nt] = mfma_f16(a, vfrag[nt][ks], accY[nt]);
+        }
+        {
+            const long long grow0 = rr.row0 + sub0 + c * CH;
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = SUB * wave + rl + r;
+                    if (row < nrows)
+                        (out + (grow0 + row) * out_stride + h * DV + NV * vb + SUB * nt)[(unsigned)cl] = f2bf(accY[nt][r]);
+                }
+        }
+        // S <- e^{G_last} S + Kg^T V'
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+            const float4 e = *reinterpret_cast<const float4*>(El + 32 * wave + SUB * mt + rl);
+            const float ev[4] = {e.x, e.y, e.z, e.w};
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) accS[mt][nt][r] *= ev[r];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const uint4 a = frag(Kl, LD64, 32 * wave + SUB * mt, 32 * ks, lane);
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt) accS[mt][nt] = mfma_f16(a, vfrag[nt][ks], accS[mt][nt]);
+            }
+        }
+        if constexpr (sizeof(S) == 2) {
+            // a bf16 state is rounded at the end of every chunk, so the result does not depend on where passes end
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) accS[mt][nt][r] = bfround(accS[mt][nt][r]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+            store_state_elem4(state_out + sbase + (long long)(NV * vb + SUB * nt + cl) * DK + 32 * wave + SUB * mt + rl,
+                              accS[mt][nt]);
+}
+
+// The gated RMSNorm over the bf16 read-outs the inter pass left in `out` (reference: kda_prefill.cu:542-570,
+// cpu.rs:361-376): a wave per (row, head), two values per lane.
+__global__ void __launch_bounds__(THREADS) norm_kernel(int H, const int32_t* __restrict__ cu_rows, int rows1,
+                                                       const bf16_t* __restrict__ G, long long g_stride,
+                                                       const bf16_t* __restrict__ norm_w, float eps, bf16_t* out,
+                                                       long long out_stride) {
+    const RowRange rr = request_rows(cu_rows, blockIdx.y, rows1);
+    const long long tasks = (long long)rr.rows * H;
+    const int wpb = THREADS / 64, lane = threadIdx.x & 63;
+    const uint32_t wpair = reinterpret_cast<const uint32_t*>(norm_w)[lane];
+    const float w0 = __uint_as_float(wpair << 16), w1 = __uint_as_float(wpair & 0xffff0000u);
+    for (long long task = (long long)blockIdx.x * wpb + (threadIdx.x >> 6); task < tasks;
+         task += (long long)gridDim.x * wpb) {
+        const long long r = rr.row0 + task / H;
+        const int h = (int)(task % H);
+        uint32_t* o = reinterpret_cast<uint32_t*>(out + r * out_stride + h * DV);
+        const uint32_t yy = o[lane];
+        const uint32_t gg = reinterpret_cast<const uint32_t*>(G + r * g_stride + h * DV)[lane];
+        const float y0 = __uint_as_float(yy << 16), y1 = __uint_as_float(yy & 0xffff0000u);
+        float ss = __builtin_fmaf(y1, y1, y0 * y0);
+        ss = ss + lane_xor16<1>(ss);
+        ss = ss + lane_xor16<2>(ss);
+        ss = ss + lane_xor16<4>(ss);
+        ss = ss + lane_xor16<8>(ss);
+        ss = ss + __shfl_xor(ss, 16, 64);
+        ss = ss + __shfl_xor(ss, 32, 64);
+        const float rinv = __builtin_amdgcn_rsqf(ss * (1.0f / (float)DV) + eps);
+        const float g0 = __uint_as_float(gg << 16), g1 = __uint_as_float(gg & 0xffff0000u);
+        o[lane] = f2bf2(w0 * (y0 * rinv) * fast_sigmoid(g0), w1 * (y1 * rinv) * fast_sigmoid(g1));
+    }
+}
+
+// Advance each request's conv window past all its rows, in place (reference: kda_prefill.cu:574-590): each lane
+// reads its three values before writing them.
+__global__ void conv_advance_kernel(int C, const int32_t* __restrict__ cu_rows, int rows1, bf16_t* conv,
+                                    const long long* __restrict__ conv_off, const bf16_t* __restrict__ P,
+                                    long long p_stride) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const RowRange rr = request_rows(cu_rows, blockIdx.y, rows1);
+    bf16_t* win = conv + (conv_off != nullptr ? conv_off[blockIdx.y] : 0);
+    bf16_t x[WINDOW];
+#pragma unroll
+    for (int j = 0; j < WINDOW; ++j) {
+        const long long src = (long long)rr.rows + j;
+        x[j] = src < WINDOW ? win[src * C + c] : P[(rr.row0 + src - WINDOW) * p_stride + c];
+    }
+#pragma unroll
+    for (int j = 0; j < WINDOW; ++j) win[(long long)j * C + c] = x[j];
+}
+
+inline const bf16_t* bfp(const glm53f_bf16* x) { return reinterpret_cast<const bf16_t*>(x); }
+inline bf16_t* bfp(glm53f_bf16* x) { return reinterpret_cast<bf16_t*>(x); }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr int kNormBlocks = 1024;
+
+// The passes over every sub-segment, the norm and the conv-window advance, in stream order (reference:
+// kda_prefill.cu:630-691).
+template <typename S>
+int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, int32_t max_rows, const glm53f_bf16* p,
+           int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g,
+           int64_t g_stride, glm53f_bf16* conv, const int64_t* conv_off, const glm53f_bf16* conv_w, const S* state_in,
+           S* state_out, const int64_t* state_off, const float* a_log, const float* dt_bias,
+           const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out, int64_t out_stride,
+           int32_t value_blocks, float* workspace, int64_t workspace_bytes, glm53f_stream_t stream) {
+    if (heads < 1 || heads > 65535 || batch < 1 || batch > 65535 || rows1 < 0 || max_rows < 0 || !p || !a || !g ||
+        !conv || !conv_w || !state_in || !state_out || !a_log || !dt_bias || !norm_w || !out || !workspace)
+        return kInvalid;
+    // Fifteen rows of decay must stay above the smallest normal f32 in a sub-chunk's products.
+    if (!(lower >= -5.8f && lower <= 0.0f)) return kInvalid;
+    if (value_blocks != 0 && value_blocks != 1 && value_blocks != 2 && value_blocks != 4) return kInvalid;
+    // 128-bit accesses to the workspace and the states, 64-bit to the conv weights, 32-bit to g and out rows.
+    if (!aligned16(workspace) || !aligned16(state_in) || !aligned16(state_out)) return kInvalid;
+    if ((reinterpret_cast<uintptr_t>(conv_w) & 7u) || (reinterpret_cast<uintptr_t>(out) & 3u) ||
+        (reinterpret_cast<uintptr_t>(g) & 3u) || (out_stride & 1) || (g_stride & 1))
+        return kInvalid;
+    (void)value_blocks;   // every accepted value runs the 32-column blocks of this build
+    const long long per_chunk = (long long)WS_BYTES * heads * batch;
+    long long chunks = workspace_bytes / per_chunk;
+    if (chunks < 1) return kInvalid;
+    const long long needed = ((long long)max_rows + CH - 1) / CH;
+    if (chunks > needed) chunks = needed > 0 ? needed : 1;
+    if (chunks > 65535) chunks = 65535;
+    hipStream_t st = (hipStream_t)stream;
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&intra_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                INTRA_LDS) != hipSuccess ||
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&inter_kernel<float>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, INTER_LDS) != hipSuccess ||
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&inter_kernel<bf16_t>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, INTER_LDS) != hipSuccess)
+            return (int)hipGetLastError();
+        attr_set = true;
+    }
+    const long long* coff = reinterpret_cast<const long long*>(conv_off);
+    const long long* soff = reinterpret_cast<const long long*>(state_off);
+    unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
+    const int step = (int)chunks * CH;
+    for (int sub0 = 0; sub0 == 0 || sub0 < max_rows; sub0 += step) {
+        if (max_rows > 0) {
+            intra_kernel<<<dim3((unsigned)chunks, heads, batch), THREADS, INTRA_LDS, st>>>(
+                heads, cu_rows, rows1, sub0, (int)chunks, bfp(p), p_stride, b_off, bfp(a), a_stride, bfp(conv), coff,
+                bfp(conv_w), a_log, dt_bias, lower, ws);
+            const int rc = (int)hipGetLastError();
+            if (rc != 0) return rc;
+        }
+        const S* s_in = sub0 == 0 ? state_in : state_out;
+        inter_kernel<S><<<dim3(heads * VBLOCKS, batch), THREADS, INTER_LDS, st>>>(
+            heads, cu_rows, rows1, sub0, (int)chunks, s_in, state_out, soff, bfp(out), out_stride, ws);
+        const int rc = (int)hipGetLastError();
+        if (rc != 0) return rc;
+        if (max_rows == 0) break;
+    }
+    if (max_rows > 0) {
+        norm_kernel<<<dim3(kNormBlocks, batch), THREADS, 0, st>>>(heads, cu_rows, rows1, bfp(g), g_stride, bfp(norm_w),
+                                                                  eps, bfp(out), out_stride);
+        const int rc = (int)hipGetLastError();
+        if (rc != 0) return rc;
+    }
+    const int C = 3 * heads * DK;
+    conv_advance_kernel<<<dim3((C + 255) / 256, batch), 256, 0, st>>>(C, cu_rows, rows1, bfp(conv), coff, bfp(p),
+                                                                      p_stride);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+}  // namespace kda
+
+using namespace kda;
+
+extern "C" int64_t glm53f_kda_prefill_workspace_bytes(int32_t heads, int32_t batch, int32_t rows_per_pass) {
+    if (heads < 1 || batch < 1 || rows_per_pass < 1) return 0;
+    return (((int64_t)rows_per_pass + CH - 1) / CH) * WS_BYTES * (int64_t)heads * batch;
+}
+
+extern "C" int glm53f_kda_prefill(int32_t heads, int32_t rows, const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
+                                  const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g, int64_t g_stride,
+                                  glm53f_bf16* conv, const glm53f_bf16* conv_w, const float* state_in,
+                                  float* state_out, const float* a_log, const float* dt_bias,
+                                  const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out,
+                                  int64_t out_stride, int32_t value_blocks, float* workspace,
+                                  int64_t workspace_bytes, glm53f_stream_t stream) {
+    return launch<float>(heads, 1, nullptr, rows, rows, p, p_stride, b_off, a, a_stride, g, g_stride, conv, nullptr,
+                         conv_w, state_in, state_out, nullptr, a_log, dt_bias, norm_w, eps, lower, out, out_stride,
+                         value_blocks, workspace, workspace_bytes, stream);
+}
+
+extern "C" int glm53f_kda_prefill_batch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t max_rows,
+                                        const glm53f_bf16* p, int64_t p_stride, int64_t b_off, const glm53f_bf16* a,
+                                        int64_t a_stride, const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv,
+                                        const int64_t* conv_off, const glm53f_bf16* conv_w, const float* state_in,
+                                        float* state_out, const int64_t* state_off, const float* a_log,
+                                        const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower,
+                                        glm53f_bf16* out, int64_t out_stride, int32_t value_blocks, float* workspace,
+                                        int64_t workspace_bytes, glm53f_stream_t stream) {
+    if (!cu_rows || !conv_off || !state_off) return kInvalid;
+    return launch<float>(heads, batch, cu_rows, 0, max_rows, p, p_stride, b_off, a, a_stride, g, g_stride, conv,
+                         conv_off, conv_w, state_in, state_out, state_off, a_log, dt_bias, norm_w, eps, lower, out,
+                         out_stride, value_blocks, workspace, workspace_bytes, stream);
+}
+
+extern "C" int glm53f_kda_prefill_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,
+                                                  int32_t max_rows, const glm53f_bf16* p, int64_t p_stride,
+                                                  int64_t b_off, const glm53f_bf16* a, int64_t a_stride,
+                                                  const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv,
+                                                  const int64_t* conv_off, const glm53f_bf16* conv_w,
+                                                  const glm53f_bf16* state_in, glm53f_bf16* state_out,
+                                                  const int64_t* state_off, const float* a_log,
+                                                  const float* dt_bias, const glm53f_bf16* norm_w, float eps,
+                                                  float lower, glm53f_bf16* out, int64_t out_stride,
+                                                  int32_t value_blocks, float* workspace, int64_t workspace_bytes,
+                                                  glm53f_stream_t stream) {
+    if (!cu_rows || !conv_off || !state_off) return kInvalid;
+    return launch<bf16_t>(heads, batch, cu_rows, 0, max_rows, p, p_stride, b_off, a, a_stride, g, g_stride, conv,
+                          conv_off, conv_w, bfp(state_in), bfp(state_out), state_off, a_log, dt_bias, norm_w, eps,
+                          lower, out, out_stride, value_blocks, workspace, workspace_bytes, stream);
 }

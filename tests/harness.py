@@ -257,3 +257,42 @@ def ulps(a, b):
 
 def bits(x):
     return np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+
+
+def prefill_batch_gpu(p: o.LayerParams, pool: Pool, slots: list[int], reqs: list[o.Rows], *, rows_per_pass=1024,
+                      value_blocks=0, write="inplace", pad=0, ws_batch=None):
+    """glm53f_kda_prefill_batch[_bf16state] over requests living in `slots` of `pool` (states and conv windows;
+    the windows are advanced in place). Returns (out rows, state tensor, meta)."""
+    w = Weights(p)
+    sr = StagedRows(stack_rows(reqs), pad=pad)
+    meta = BatchMeta([r.rows for r in reqs], [pool.conv_off(s) for s in slots], [pool.state_off(s) for s in slots])
+    nb = ws_batch or meta.batch
+    ws_bytes = ffi.glm53f_kda_prefill_workspace_bytes(p.heads, nb, rows_per_pass)
+    assert ws_bytes > 0
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=DEV)
+    s_out = pool.state if write == "inplace" else torch.zeros_like(pool.state)
+    fn = ffi.glm53f_kda_prefill_batch_bf16state if pool.bf16 else ffi.glm53f_kda_prefill_batch
+    code = fn(p.heads, meta.batch, ptr(meta.cu_rows), max(meta.rows), *sr.row_args(), ptr(pool.conv),
+              ptr(meta.conv_off), ptr(w.conv_w), ptr(pool.state), ptr(s_out), ptr(meta.state_off), *w.args(),
+              ptr(sr.out), sr.out_stride, value_blocks, ptr(ws), ws_bytes, None)
+    check(code, "prefill_batch")
+    sync()
+    return sr.out_np(), s_out, meta
+
+
+def prefill_gpu(p: o.LayerParams, conv: np.ndarray, state: np.ndarray, rows: o.Rows, *, rows_per_pass=1024,
+                value_blocks=0, in_place=False, pad=0, b_first=False):
+    """glm53f_kda_prefill on one request, f32 state. Returns (out, state, conv window after)."""
+    w = Weights(p)
+    sr = StagedRows(rows, pad=pad, b_first=b_first)
+    conv_d = to_bf16(conv)
+    s_in = to_f32(state)
+    s_out = s_in if in_place else torch.zeros_like(s_in)
+    ws_bytes = ffi.glm53f_kda_prefill_workspace_bytes(p.heads, 1, rows_per_pass)
+    ws = torch.empty(max(ws_bytes, 16) // 4, dtype=torch.float32, device=DEV)
+    code = ffi.glm53f_kda_prefill(p.heads, rows.rows, *sr.row_args(), ptr(conv_d), ptr(w.conv_w), ptr(s_in),
+                                  ptr(s_out), *w.args(), ptr(sr.out), sr.out_stride, value_blocks, ptr(ws), ws_bytes,
+                                  None)
+    check(code, "prefill")
+    sync()
+    return sr.out_np(), back(s_out), back(conv_d)
