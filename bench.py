@@ -186,6 +186,110 @@ def bench_decode(steps, warmup, stream, cpu=True):
     return res
 
 
+# ------------------------------------------------------------------------------------------------ prefill
+
+def bench_prefill(steps, warmup, stream, cpu=True):
+    """BASELINE config 2: one prompt of 8192 rows as four sequential calls of 2048 rows on one slot (the
+    engine's lanes), 64 heads, f32 carried state, conv and output gate included."""
+    heads, total, lane_rows = HEADS, 8192, 2048
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    layer = Layer(heads, gen)
+    n, cw = state_len(heads), WINDOW * channels(heads)
+    rows = RowBuffers(heads, total, gen)
+    state = torch.zeros(n, device=DEV)
+    conv = torch.randn(cw, device=DEV, generator=gen).to(torch.bfloat16)
+    ws_bytes = ffi.glm53f_kda_prefill_workspace_bytes(heads, 1, lane_rows)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=DEV)
+    st = stream.cuda_stream
+    fn = ffi.glm53f_kda_prefill
+    calls = [(heads, lane_rows, *rows.row_args(first), ptr(conv), ptr(layer.conv_w), ptr(state), ptr(state),
+              *layer.args(), *rows.out_args(first), 0, ptr(ws), ws_bytes, st) for first in range(0, total, lane_rows)]
+
+    def step():
+        for a in calls:
+            check(fn(*a), "prefill")
+
+    ms = timed(step, steps, warmup, stream)
+    flops = total * 11_709_099 / 64 * heads        # dense MFMA count of the chunk-64 form: 11.71 MFLOP per token
+    io_bytes = total * 98_432                       # compulsory row traffic: p, a, g in, out
+    res = {
+        "tok_per_s_per_layer": total / (ms * 1e-3), "ms_per_8192_tokens": ms,
+        "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "prefill (intra + inter + norm + conv advance, whole call)",
+                     "flops_per_token": 11_709_099, "hbm_GBps_compulsory": io_bytes / (ms * 1e-3) / 1e9,
+                     "hbm_frac": io_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+        "config": {"workload": "BASELINE config 2: T=8192 as 4 calls of 2048 rows on one slot, H=64, chunk 64, "
+                               "bf16 rows, f32 state, conv + output gate", "workspace_MB": ws_bytes / 1e6},
+    }
+    if cpu:
+        from oracle import kda_oracle as o
+        threads = min(16, os.cpu_count() or 1)
+        sample = 256
+        p = o.LayerParams(heads, layer.conv_w.float().cpu().numpy(), layer.a_log.cpu().numpy(),
+                          layer.dt_bias.cpu().numpy(), layer.norm_w.float().cpu().numpy())
+        rq = rows.to_oracle(o, 0, sample)
+        conv0 = conv.float().cpu().numpy()
+        s0 = np.zeros(n, np.float32)
+        t0 = time.perf_counter()
+        o.literal_chain(p, conv0, s0, rq, threads=threads)
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": sample / dt, "unit": "tok/s per layer", "cores": threads, "kind": "port",
+                               "sample": f"the first {sample} rows of the prompt, 64 heads, the C oracle's literal "
+                                         f"recurrent chain (conv, gates, delta rule, gated norm), {dt:.2f} s"}
+    return res
+
+
+# ------------------------------------------------------------------------------------------------ verify
+
+def bench_verify(steps, warmup, stream):
+    """BASELINE config 4: 48 slots x 16 draft rows, bf16 state, a checkpoint after every row, then the commit by
+    selection with an accepted length per slot drawn uniformly from [0, 16]."""
+    heads, slots_n, drafts, layers = HEADS, 48, 16, 2
+    gen = torch.Generator(device=DEV).manual_seed(4)
+    layer = Layer(heads, gen)
+    n, cw = state_len(heads), WINDOW * channels(heads)
+    pools = (torch.randn(layers, slots_n * n, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
+    convs = torch.randn(layers, slots_n * cw, device=DEV, generator=gen).to(torch.bfloat16)
+    rows = RowBuffers(heads, slots_n * drafts, gen)
+    ck = torch.empty(layers, slots_n * drafts * n, dtype=torch.bfloat16, device=DEV)
+    cu = (torch.arange(slots_n + 1, dtype=torch.int32) * drafts).to(DEV)
+    keep = torch.randint(0, drafts + 1, (slots_n,), generator=torch.Generator().manual_seed(5)).to(torch.int32).to(DEV)
+    soff = (torch.arange(slots_n, dtype=torch.int64) * n).to(DEV)
+    coff = (torch.arange(slots_n, dtype=torch.int64) * cw).to(DEV)
+    st = stream.cuda_stream
+    vfn, sfn = ffi.glm53f_kda_verify_batch_bf16state, ffi.glm53f_kda_select_batch_bf16state
+    vargs = [(heads, slots_n, ptr(cu), *rows.row_args(), ptr(convs[l]), ptr(coff), ptr(layer.conv_w), ptr(pools[l]),
+              ptr(soff), *layer.args(), *rows.out_args(), ptr(ck[l]), None, None, None, None, st)
+             for l in range(layers)]
+    sargs = [(heads, 1, slots_n, ptr(cu), ptr(keep), ptr(ck[l]), 0, ptr(pools[l]), 0, ptr(soff), st)
+             for l in range(layers)]
+    it = [0]
+
+    def verify():
+        check(vfn(*vargs[it[0] % layers]), "verify")
+        it[0] += 1
+
+    def select():
+        check(sfn(*sargs[it[0] % layers]), "select")
+        it[0] += 1
+
+    ms_v = timed(verify, steps, warmup, stream)
+    ms_s = timed(select, steps, warmup, stream)
+    vbytes = slots_n * n * 2 + slots_n * drafts * n * 2          # read 48 states + write 48 x 16 checkpoints
+    kept = int((keep > 0).sum().item())
+    sbytes = 2 * kept * n * 2
+    return {
+        "verify_ms_per_layer": ms_v, "select_ms_per_layer": ms_s,
+        "roofline": {"bound": "hbm", "achieved": vbytes / (ms_v * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": vbytes / (ms_v * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "chain_kernel<bf16> with checkpoints", "bytes_per_launch": vbytes},
+        "select_GBps": sbytes / (ms_s * 1e-3) / 1e9,
+        "config": {"workload": "BASELINE config 4: verify 48 slots x 16 drafts, bf16 state, per-row checkpoints; "
+                               "select with keep ~ U{0..16}", "kept_slots": kept},
+    }
+
+
 # ------------------------------------------------------------------------------------------------ main
 
 def main():
@@ -218,6 +322,19 @@ def main():
                                 "slots": 16, "pool_slots": 48, "heads": 64, "layers": 34}})
         if "cpu_baseline" in dec:
             line["cpu_baseline"] = dec["cpu_baseline"]
+    if args.only in (None, "prefill"):
+        pre = bench_prefill(max(2, args.steps // 4), max(1, args.warmup // 2), stream, cpu=not args.no_cpu)
+        line["prefill"] = pre
+        if args.only == "prefill":
+            line.update({"value": pre["tok_per_s_per_layer"], "unit": "tok/s per layer",
+                         "ms_per_step": pre["ms_per_8192_tokens"], "roofline": pre["roofline"],
+                         "config": pre["config"]})
+    if args.only in (None, "verify"):
+        ver = bench_verify(max(2, args.steps // 4), max(1, args.warmup // 2), stream)
+        line["verify"] = ver
+        if args.only == "verify":
+            line.update({"value": ver["roofline"]["achieved"], "ms_per_step": ver["verify_ms_per_layer"],
+                         "roofline": ver["roofline"], "config": ver["config"]})
     print(json.dumps(line))
 
 

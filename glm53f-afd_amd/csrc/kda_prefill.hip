@@ -32,6 +32,7 @@ typedef _Float16 f16_t;
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // a register-friendly 128-bit piece
 
 // Workspace of one (request, head, chunk), bytes.
 constexpr int WS_W = 0;                   // fp16 [64 rows][128 keys]
@@ -115,17 +116,55 @@ constexpr int I_END = I_R1 + 2 * P_ROWS32;
 constexpr int I_T = I_PASS;                       // f32 [64][LDF]
 constexpr int I_X = I_T + CH * LDF * 4;           // f32 [64][LDF]
 constexpr int I_TQ = I_X + CH * LDF * 4;          // fp16 [64][LD64]: T diag(beta)
+// Input staging (before the operands of a half land): the half's 35 rows of q | k | v, and the chunk's gate rows.
+constexpr int LDX = DK + 8;                       // staged input rows, 16-bit elements
+constexpr int XROWS = 32 + WINDOW;
+constexpr int I_XIN = I_R2;                       // bf16 [3][35][LDX]
+constexpr int I_AIN = I_PASS;                     // bf16 [64][LDX]
+static_assert(I_XIN + 3 * XROWS * LDX * 2 <= I_END, "input staging must fit behind the diagonal operands");
 constexpr int INTRA_LDS = I_END;
 static_assert(I_TQ + CH * LD64 * 2 <= I_END, "inverse scratch must fit the per-half region");
 static_assert(INTRA_LDS <= 160 * 1024, "intra_kernel LDS");
 
+// Copy NROWS rows of 128 bf16 from global memory into LDS rows of LDX elements. src(row) is the row's address or
+// nullptr for a row of zeros. With `vec` every row is 16-byte aligned and moves in 128-bit pieces; all loads of a
+// lane are issued before the first store, so a lane waits for one memory latency, not one per row.
+template <int NROWS, typename F>
+__device__ __forceinline__ void stage_rows(uint16_t* dst, F src, bool vec, int t) {
+    if (vec) {
+        constexpr int PIECES = NROWS * 16, IT = (PIECES + THREADS - 1) / THREADS;
+        u32x4 x[IT];
+#pragma unroll
+        for (int q = 0; q < IT; ++q) {
+            const int v = q * THREADS + t, row = v >> 4;
+            const bf16_t* p = v < PIECES ? src(row) : nullptr;
+            x[q] = p != nullptr ? *reinterpret_cast<const u32x4*>(p + (v & 15) * 8) : u32x4{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int q = 0; q < IT; ++q) {
+            const int v = q * THREADS + t;
+            if (v < PIECES) *reinterpret_cast<u32x4*>(dst + (v >> 4) * LDX + (v & 15) * 8) = x[q];
+        }
+    } else {
+        constexpr int ELEMS = NROWS * DK, IT = (ELEMS + THREADS - 1) / THREADS;
+#pragma unroll 8
+        for (int q = 0; q < IT; ++q) {
+            const int e = q * THREADS + t, row = e >> 7;
+            if (e < ELEMS) {
+                const bf16_t* p = src(row);
+                dst[row * LDX + (e & 127)] = p != nullptr ? p[e & 127] : (bf16_t)0;
+            }
+        }
+    }
+}
+
 // Pass 1: one chunk of one head of one request, everything that does not need the state, into its workspace slot.
-__global__ void __launch_bounds__(THREADS) intra_kernel(
+__global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) intra_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
         const bf16_t* __restrict__ P, long long p_stride, long long b_off, const bf16_t* __restrict__ A,
         long long a_stride, const bf16_t* __restrict__ conv, const long long* __restrict__ conv_off,
         const bf16_t* __restrict__ cw, const float* __restrict__ a_log, const float* __restrict__ dt_bias, float lower,
-        unsigned char* __restrict__ ws) {
+        int vec, unsigned char* __restrict__ ws) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const RowRange rr = request_rows(cu_rows, b, rows1);
@@ -147,6 +186,11 @@ __global__ void __launch_bounds__(THREADS) intra_kernel(
     uint16_t* KC1 = reinterpret_cast<uint16_t*>(smem + I_KC1);
 
     // ---- gates of the whole chunk: cumulative log decay of this lane's channel inside its two sub-chunks
+    uint16_t* ain = reinterpret_cast<uint16_t*>(smem + I_AIN);
+    stage_rows<CH>(ain, [&](int R) -> const bf16_t* {
+        return R < n ? A + (rr.row0 + r0 + R) * a_stride + h * DK : nullptr;
+    }, vec != 0, t);
+    __syncthreads();
     const float rate = fast_exp(a_log[h]);
     const float dtb = dt_bias[h * DK + d];
     float cg[2][SUB];                             // inclusive cumulative sums, sub-chunks s and 2 + s
@@ -158,10 +202,7 @@ __global__ void __launch_bounds__(THREADS) intra_kernel(
         for (int i = 0; i < SUB; ++i) {
             const int R = SUB * a + i;
             float g = 0.0f;
-            if (R < n) {
-                const float av = bf2f((A + (rr.row0 + r0 + R) * a_stride + h * DK)[(unsigned)d]);
-                g = lower * fast_sigmoid(rate * (av + dtb));
-            }
+            if (R < n) g = lower * fast_sigmoid(rate * (bf2f(ain[R * LDX + d]) + dtb));
             run += g;
             cg[h2][i] = run;
         }
@@ -194,30 +235,43 @@ __global__ void __launch_bounds__(THREADS) intra_kernel(
     for (int a = 0; a < 4; ++a) Bp[a + 1] = Bp[a] + tot[a * DK + d];
     if (s == 0) reinterpret_cast<float*>(wsc + WS_E)[d] = fast_exp(Bp[4]);
 
-    // Row `rel` (relative to the request's first row; -3..-1 are the conv window) of channel ch, 0 past the end.
-    auto input = [&](int rel, unsigned ch) -> float {
-        if (rel >= rr.rows) return 0.0f;
-        const bf16_t* src = rel < 0 ? cs + (long long)(rel + WINDOW) * C : P + (rr.row0 + rel) * p_stride;
-        return bf2f(src[ch]);
+    // Row `rel` (relative to the request's first row; -3..-1 are the conv window) of q | k | v, nullptr past the end.
+    auto input_row = [&](int rel) -> const bf16_t* {
+        if (rel >= rr.rows) return nullptr;
+        return rel < 0 ? cs + (long long)(rel + WINDOW) * C : P + (rr.row0 + rel) * p_stride;
     };
 
-    // ---- the two halves of the chunk: sub-chunks {0, 1}, then {2, 3}
-#pragma unroll 1
+    // ---- the two halves of the chunk: sub-chunks {0, 1}, then {2, 3} (unrolled: h2 indexes registers)
+#pragma unroll
     for (int h2 = 0; h2 < 2; ++h2) {
         const int a = 2 * h2 + s;                 // this lane's sub-chunk
         const int lr0 = SUB * s;                  // its first row inside the half's 32-row arrays
         uint16_t* rawq = reinterpret_cast<uint16_t*>(smem + I_RAWQ);
         uint16_t* rawk = reinterpret_cast<uint16_t*>(smem + I_RAWK);
+        // the half's input rows (three before its first row included) into LDS, q | k | v side by side
+        uint16_t* xin = reinterpret_cast<uint16_t*>(smem + I_XIN);
+        {
+            const int first = r0 + 32 * h2 - WINDOW;
+#pragma unroll
+            for (int seg = 0; seg < 3; ++seg)
+                stage_rows<XROWS>(xin + seg * XROWS * LDX, [&](int j) -> const bf16_t* {
+                    const bf16_t* row = input_row(first + j);
+                    return row != nullptr ? row + seg * H * DK + h * DK : nullptr;
+                }, vec != 0, t);
+        }
+        __syncthreads();
         // conv + SiLU, one bf16 rounding, 16 rows of q, k, v
         float qr[SUB], kr[SUB];
         {
-            const int rel0 = r0 + SUB * a;
+            const uint16_t* xq_l = xin + (SUB * s) * LDX + d;                 // row j of the lane's sub-chunk: + j * LDX
+            const uint16_t* xk_l = xq_l + XROWS * LDX;
+            const uint16_t* xv_l = xk_l + XROWS * LDX;
             float xq[TAPS], xk[TAPS], xv[TAPS];
 #pragma unroll
             for (int j = 0; j < WINDOW; ++j) {
-                xq[j + 1] = input(rel0 - WINDOW + j, cq);
-                xk[j + 1] = input(rel0 - WINDOW + j, ck);
-                xv[j + 1] = input(rel0 - WINDOW + j, cv);
+                xq[j + 1] = bf2f(xq_l[j * LDX]);
+                xk[j + 1] = bf2f(xk_l[j * LDX]);
+                xv[j + 1] = bf2f(xv_l[j * LDX]);
             }
             uint32_t vpack[SUB / 2];
 #pragma unroll
@@ -225,9 +279,9 @@ __global__ void __launch_bounds__(THREADS) intra_kernel(
 #pragma unroll
                 for (int j = 0; j < WINDOW; ++j) { xq[j] = xq[j + 1]; xk[j] = xk[j + 1]; xv[j] = xv[j + 1]; }
                 const bool live = SUB * a + i < n;
-                xq[3] = live ? input(rel0 + i, cq) : 0.0f;
-                xk[3] = live ? input(rel0 + i, ck) : 0.0f;
-                xv[3] = live ? input(rel0 + i, cv) : 0.0f;
+                xq[3] = bf2f(xq_l[(WINDOW + i) * LDX]);
+                xk[3] = bf2f(xk_l[(WINDOW + i) * LDX]);
+                xv[3] = bf2f(xv_l[(WINDOW + i) * LDX]);
                 float aq = 0.0f, ak = 0.0f, av = 0.0f;
 #pragma unroll
                 for (int tap = 0; tap < TAPS; ++tap) {
@@ -518,7 +572,7 @@ __device__ __forceinline__ void store_state_elem4(bf16_t* p, const f32x4 v) {
 // Pass 2: one head's NV value columns of one request through the chunks of the pass, in order. The state
 // S[128 keys][NV] lives in MFMA accumulators: wave w owns keys 32 w .. 32 w + 31.
 template <typename S>
-__global__ void __launch_bounds__(THREADS) inter_kernel(
+__global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) inter_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
         const S* state_in, S* state_out, const long long* __restrict__ state_off,
         bf16_t* __restrict__ out, long long out_stride, const unsigned char* __restrict__ ws) {
@@ -553,41 +607,39 @@ __global__ void __launch_bounds__(THREADS) inter_kernel(
         }
 
     const unsigned char* wsh = ws + ((long long)b * H + h) * chunks * (long long)WS_BYTES;
-    // Staging of a chunk's workspace: global -> registers (issued a chunk ahead) -> LDS.
-    uint4 stage[STAGE_PER_LANE];
-    auto stage_load = [&](int c) {
-        const unsigned char* src = wsh + (long long)c * WS_BYTES;
-#pragma unroll
-        for (int q = 0; q < STAGE_PER_LANE; ++q) {
-            const int v = q * THREADS + t;
-            if (v < STAGE_VEC) {
-                int off;   // piece index -> byte offset in the workspace
-                if (v < 1024) off = WS_W + v * 16;
-                else if (v < 2048) off = WS_QG + (v - 1024) * 16;
-                else if (v < 3072) off = WS_KGT + (v - 2048) * 16;
-                else if (v < 3584) off = WS_M + (v - 3072) * 16;
-                else if (v < 3584 + NV * CH / 8) off = WS_UT + NV * vb * CH * 2 + (v - 3584) * 16;
-                else off = WS_E + (v - 3584 - NV * CH / 8) * 16;
-                stage[q] = *reinterpret_cast<const uint4*>(src + off);
-            }
-        }
-    };
-    auto stage_store = [&]() {
-#pragma unroll
-        for (int q = 0; q < STAGE_PER_LANE; ++q) {
-            const int v = q * THREADS + t;
-            if (v < STAGE_VEC) {
-                unsigned char* dst;
-                if (v < 1024) dst = smem + N_W + ((v >> 4) * LD128 + (v & 15) * 8) * 2;                 // 16 pieces per row
-                else if (v < 2048) dst = smem + N_Q + (((v - 1024) >> 4) * LD128 + ((v - 1024) & 15) * 8) * 2;
-                else if (v < 3072) dst = smem + N_K + (((v - 2048) >> 3) * LD64 + ((v - 2048) & 7) * 8) * 2;  // 8 per row
-                else if (v < 3584) dst = smem + N_M + (((v - 3072) >> 3) * LD64 + ((v - 3072) & 7) * 8) * 2;
-                else if (v < 3584 + NV * CH / 8) dst = smem + N_U + (((v - 3584) >> 3) * LD64 + ((v - 3584) & 7) * 8) * 2;
-                else dst = smem + N_E + (v - 3584 - NV * CH / 8) * 16;
-                *reinterpret_cast<uint4*>(dst) = stage[q];
-            }
-        }
-    };
+    // Staging of a chunk's workspace: global -> registers (issued a chunk ahead) -> LDS. Every piece index q
+    // has its own array, so source and destination are compile-time functions of q: W (q 0-3), Qg (4-7),
+    // Kg^T (8-11), M (12-13), this block's rows of U^T (14), e^{G_last} (15, 32 lanes).
+    static_assert(STAGE_PER_LANE == 16 && NV == 32, "staging map");
+    u32x4 stage[STAGE_PER_LANE];
+    const unsigned stage_lo = (unsigned)t * 16u;
+#define KDA_STAGE_LOAD(C_)                                                                                          \
+    {                                                                                                               \
+        const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                               \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                                             \
+            stage[q] = *reinterpret_cast<const u32x4*>(src_ + WS_W + q * 4096 + stage_lo);                           \
+            stage[4 + q] = *reinterpret_cast<const u32x4*>(src_ + WS_QG + q * 4096 + stage_lo);                      \
+            stage[8 + q] = *reinterpret_cast<const u32x4*>(src_ + WS_KGT + q * 4096 + stage_lo);                     \
+        }                                                                                                           \
+        stage[12] = *reinterpret_cast<const u32x4*>(src_ + WS_M + stage_lo);                                        \
+        stage[13] = *reinterpret_cast<const u32x4*>(src_ + WS_M + 4096 + stage_lo);                                 \
+        stage[14] = *reinterpret_cast<const u32x4*>(src_ + WS_UT + NV * vb * CH * 2 + stage_lo);                    \
+        stage[15] = *reinterpret_cast<const u32x4*>(src_ + WS_E + (stage_lo & 511u));                               \
+    }
+    // 128-wide rows take 16 pieces each, 64-wide rows 8
+#define KDA_STAGE_STORE()                                                                                           \
+    {                                                                                                               \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                                             \
+            const int v_ = q * THREADS + t;                                                                         \
+            *reinterpret_cast<u32x4*>(Wl + (v_ >> 4) * LD128 + (v_ & 15) * 8) = stage[q];                            \
+            *reinterpret_cast<u32x4*>(Ql + (v_ >> 4) * LD128 + (v_ & 15) * 8) = stage[4 + q];                        \
+            *reinterpret_cast<u32x4*>(Kl + (v_ >> 3) * LD64 + (v_ & 7) * 8) = stage[8 + q];                          \
+        }                                                                                                           \
+        *reinterpret_cast<u32x4*>(Ml + (t >> 3) * LD64 + (t & 7) * 8) = stage[12];                                  \
+        *reinterpret_cast<u32x4*>(Ml + ((THREADS + t) >> 3) * LD64 + (t & 7) * 8) = stage[13];                      \
+        *reinterpret_cast<u32x4*>(Ul + (t >> 3) * LD64 + (t & 7) * 8) = stage[14];                                  \
+        if (t < 32) *reinterpret_cast<u32x4*>(El + t * 4) = stage[15];                                              \
+    }
     // S^T for the first chunk
     auto put_state = [&]() {
 #pragma unroll
@@ -600,13 +652,13 @@ __global__ void __launch_bounds__(THREADS) inter_kernel(
             }
     };
 
-    if (nch > 0) stage_load(0);
+    if (nch > 0) KDA_STAGE_LOAD(0)
     for (int c = 0; c < nch; ++c) {
         const int nrows = min(CH, left - c * CH);
-        stage_store();
+        KDA_STAGE_STORE()
         put_state();
         __syncthreads();
-        if (c + 1 < nch) stage_load(c + 1);
+        if (c + 1 < nch) KDA_STAGE_LOAD(c + 1)
         const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
         // V' = U - W S: wave w takes rows 16 w .. 16 w + 15
         uint4 sfrag[2][4];
@@ -795,12 +847,16 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
     const long long* coff = reinterpret_cast<const long long*>(conv_off);
     const long long* soff = reinterpret_cast<const long long*>(state_off);
     unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
+    // 128-bit input staging needs every q | k | v and gate row segment on a 16-byte boundary (the model's strides
+    // are); other layouts take the 16-bit path. Conv-window offsets are device data: whole windows keep alignment.
+    const int vec = aligned16(p) && aligned16(a) && aligned16(conv) && (p_stride % 8 == 0) && (a_stride % 8 == 0) &&
+                    (heads % 1 == 0);
     const int step = (int)chunks * CH;
     for (int sub0 = 0; sub0 == 0 || sub0 < max_rows; sub0 += step) {
         if (max_rows > 0) {
             intra_kernel<<<dim3((unsigned)chunks, heads, batch), THREADS, INTRA_LDS, st>>>(
                 heads, cu_rows, rows1, sub0, (int)chunks, bfp(p), p_stride, b_off, bfp(a), a_stride, bfp(conv), coff,
-                bfp(conv_w), a_log, dt_bias, lower, ws);
+                bfp(conv_w), a_log, dt_bias, lower, vec, ws);
             const int rc = (int)hipGetLastError();
             if (rc != 0) return rc;
         }
