@@ -126,37 +126,45 @@ constexpr int INTRA_LDS = I_END;
 static_assert(I_TQ + CH * LD64 * 2 <= I_END, "inverse scratch must fit the per-half region");
 static_assert(INTRA_LDS <= 160 * 1024, "intra_kernel LDS");
 
-// Copy NROWS rows of 128 bf16 from global memory into LDS rows of LDX elements. src(row) is the row's address or
-// nullptr for a row of zeros. With `vec` every row is 16-byte aligned and moves in 128-bit pieces; all loads of a
-// lane are issued before the first store, so a lane waits for one memory latency, not one per row.
-template <int NROWS, typename F>
-__device__ __forceinline__ void stage_rows(uint16_t* dst, F src, bool vec, int t) {
-    if (vec) {
-        constexpr int PIECES = NROWS * 16, IT = (PIECES + THREADS - 1) / THREADS;
-        u32x4 x[IT];
+// NROWS rows of 128 bf16 on their way from global memory to LDS rows of LDX elements. src(row) is the row's
+// address or nullptr for a row of zeros. With `vec` every row is 16-byte aligned and moves in 128-bit pieces:
+// load() issues all of a lane's loads at once, store() lands them later, so the memory latency hides behind
+// whatever runs in between. Without `vec` store() copies 16-bit elements directly.
+template <int NROWS>
+struct StagedRows {
+    static constexpr int PIECES = NROWS * 16, IT = (PIECES + THREADS - 1) / THREADS;
+    u32x4 x[IT];
+    template <typename F>
+    __device__ __forceinline__ void load(F src, bool vec, int t) {
+        if (!vec) return;
 #pragma unroll
         for (int q = 0; q < IT; ++q) {
             const int v = q * THREADS + t, row = v >> 4;
             const bf16_t* p = v < PIECES ? src(row) : nullptr;
             x[q] = p != nullptr ? *reinterpret_cast<const u32x4*>(p + (v & 15) * 8) : u32x4{0u, 0u, 0u, 0u};
         }
+    }
+    template <typename F>
+    __device__ __forceinline__ void store(uint16_t* dst, F src, bool vec, int t) const {
+        if (vec) {
 #pragma unroll
-        for (int q = 0; q < IT; ++q) {
-            const int v = q * THREADS + t;
-            if (v < PIECES) *reinterpret_cast<u32x4*>(dst + (v >> 4) * LDX + (v & 15) * 8) = x[q];
-        }
-    } else {
-        constexpr int ELEMS = NROWS * DK, IT = (ELEMS + THREADS - 1) / THREADS;
+            for (int q = 0; q < IT; ++q) {
+                const int v = q * THREADS + t;
+                if (v < PIECES) *reinterpret_cast<u32x4*>(dst + (v >> 4) * LDX + (v & 15) * 8) = x[q];
+            }
+        } else {
+            constexpr int ELEMS = NROWS * DK, ITE = (ELEMS + THREADS - 1) / THREADS;
 #pragma unroll 8
-        for (int q = 0; q < IT; ++q) {
-            const int e = q * THREADS + t, row = e >> 7;
-            if (e < ELEMS) {
-                const bf16_t* p = src(row);
-                dst[row * LDX + (e & 127)] = p != nullptr ? p[e & 127] : (bf16_t)0;
+            for (int q = 0; q < ITE; ++q) {
+                const int e = q * THREADS + t, row = e >> 7;
+                if (e < ELEMS) {
+                    const bf16_t* p = src(row);
+                    dst[row * LDX + (e & 127)] = p != nullptr ? p[e & 127] : (bf16_t)0;
+                }
             }
         }
     }
-}
+};
 
 // Pass 1: one chunk of one head of one request, everything that does not need the state, into its workspace slot.
 __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) intra_kernel(
@@ -186,10 +194,29 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
     uint16_t* KC1 = reinterpret_cast<uint16_t*>(smem + I_KC1);
 
     // ---- gates of the whole chunk: cumulative log decay of this lane's channel inside its two sub-chunks
-    uint16_t* ain = reinterpret_cast<uint16_t*>(smem + I_AIN);
-    stage_rows<CH>(ain, [&](int R) -> const bf16_t* {
+    // Row `rel` (relative to the request's first row; -3..-1 are the conv window) of q | k | v, nullptr past the end.
+    auto input_row = [&](int rel) -> const bf16_t* {
+        if (rel >= rr.rows) return nullptr;
+        return rel < 0 ? cs + (long long)(rel + WINDOW) * C : P + (rr.row0 + rel) * p_stride;
+    };
+    // segment seg (q, k, v) of the input rows of half h2, three rows before its first included
+    auto x_src = [&](int h2, int seg) {
+        return [=](int j) -> const bf16_t* {
+            const bf16_t* row = input_row(r0 + 32 * h2 - WINDOW + j);
+            return row != nullptr ? row + seg * H * DK + h * DK : nullptr;
+        };
+    };
+    auto a_src = [&](int R) -> const bf16_t* {
         return R < n ? A + (rr.row0 + r0 + R) * a_stride + h * DK : nullptr;
-    }, vec != 0, t);
+    };
+    // every global input of the first half goes out now; the second half's follows while the first computes
+    StagedRows<CH> a_st;
+    StagedRows<XROWS> x_st[3];
+    a_st.load(a_src, vec != 0, t);
+#pragma unroll
+    for (int seg = 0; seg < 3; ++seg) x_st[seg].load(x_src(0, seg), vec != 0, t);
+    uint16_t* ain = reinterpret_cast<uint16_t*>(smem + I_AIN);
+    a_st.store(ain, a_src, vec != 0, t);
     __syncthreads();
     const float rate = fast_exp(a_log[h]);
     const float dtb = dt_bias[h * DK + d];
@@ -235,12 +262,6 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
     for (int a = 0; a < 4; ++a) Bp[a + 1] = Bp[a] + tot[a * DK + d];
     if (s == 0) reinterpret_cast<float*>(wsc + WS_E)[d] = fast_exp(Bp[4]);
 
-    // Row `rel` (relative to the request's first row; -3..-1 are the conv window) of q | k | v, nullptr past the end.
-    auto input_row = [&](int rel) -> const bf16_t* {
-        if (rel >= rr.rows) return nullptr;
-        return rel < 0 ? cs + (long long)(rel + WINDOW) * C : P + (rr.row0 + rel) * p_stride;
-    };
-
     // ---- the two halves of the chunk: sub-chunks {0, 1}, then {2, 3} (unrolled: h2 indexes registers)
 #pragma unroll
     for (int h2 = 0; h2 < 2; ++h2) {
@@ -250,16 +271,13 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         uint16_t* rawk = reinterpret_cast<uint16_t*>(smem + I_RAWK);
         // the half's input rows (three before its first row included) into LDS, q | k | v side by side
         uint16_t* xin = reinterpret_cast<uint16_t*>(smem + I_XIN);
-        {
-            const int first = r0 + 32 * h2 - WINDOW;
 #pragma unroll
-            for (int seg = 0; seg < 3; ++seg)
-                stage_rows<XROWS>(xin + seg * XROWS * LDX, [&](int j) -> const bf16_t* {
-                    const bf16_t* row = input_row(first + j);
-                    return row != nullptr ? row + seg * H * DK + h * DK : nullptr;
-                }, vec != 0, t);
-        }
+        for (int seg = 0; seg < 3; ++seg) x_st[seg].store(xin + seg * XROWS * LDX, x_src(h2, seg), vec != 0, t);
         __syncthreads();
+        if (h2 == 0) {
+#pragma unroll
+            for (int seg = 0; seg < 3; ++seg) x_st[seg].load(x_src(1, seg), vec != 0, t);
+        }
         // conv + SiLU, one bf16 rounding, 16 rows of q, k, v
         float qr[SUB], kr[SUB];
         {

@@ -6,7 +6,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_HERE), "csrc", "libglm53f_kda.so")
+LIB_PATH = os.environ.get("GLM53F_KDA_LIB") or os.path.join(os.path.dirname(_HERE), "csrc", "libglm53f_kda.so")
 
 i32, i64, f32, ptr = C.c_int32, C.c_int64, C.c_float, C.c_void_p
 
