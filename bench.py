@@ -127,9 +127,10 @@ def bench_decode(steps, warmup, stream, cpu=True):
 
     # Argument lists are built once: the timed loops only make the C calls.
     chain_fn, shift_fn = ffi.glm53f_kda_chain_batch_bf16state, ffi.glm53f_kda_conv_shift_batch
-    chain_args = [(heads, batch, ptr(cu), *rows.row_args(), ptr(convs[l]), ptr(coff), ptr(layer.conv_w),
-                   ptr(pools[l]), ptr(pools[l]), ptr(soff), *layer.args(), *rows.out_args(), None, None, None, None,
-                   st) for l in range(layers)]
+    same = int(os.environ.get("KDA_BENCH_SAME_POOL", "0"))   # diagnostic: every layer on one pool (cache-resident)
+    chain_args = [(heads, batch, ptr(cu), *rows.row_args(), ptr(convs[0 if same else l]), ptr(coff),
+                   ptr(layer.conv_w), ptr(pools[0 if same else l]), ptr(pools[0 if same else l]), ptr(soff),
+                   *layer.args(), *rows.out_args(), None, None, None, None, st) for l in range(layers)]
     shift_args = [(c, 1, batch, ptr(cu), ptr(keep), ptr(convs[l]), 0, ptr(coff), ptr(rows.p), 0, rows.p_stride, st)
                   for l in range(layers)]
 

@@ -76,48 +76,68 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
         }
         return;
     }
-    // The state's loads go out first: their latency hides behind the first row's prologue. Between rows the
-    // state stays in its stored form (`raw`: packed bf16 pairs, or f32 bits): a bf16 state is rounded after
-    // every row anyway, and the packed form halves the registers it holds.
-    uint4 raw[M::STEPS];
-    load_state<S>(state_in + sbase, soff_lane, raw);
     const float decay_rate = expf(a_log[h]);
 
-    // A row's prologue, two items per lane: lane t takes conv channel t of q|k (q for t < 128, k after), then
-    // v channel t (t < 128) or decay channel t - 128; then the L2 norms of q and k by wave 0.
-    auto prologue = [&](int r) {
+    // A row's prologue. Every global load of the row goes out first, back to back and without branches (lanes
+    // that have no use for a value load a neighbour's and drop it), so a row pays one memory latency, not one
+    // per stage: the inputs and weights of conv channel t of q|k (q for t < 128, k after) and of v channel
+    // t % 128, the forget-gate input and bias of key channel t % 128, the beta logit, and the output gate and
+    // norm weight of value channel t % 128 for the row's epilogue.
+    const int i7 = t & (DK - 1);
+    const unsigned c0 = (unsigned)((t >> 7) * H * DK + h * DK + i7);      // q | k channel of this lane
+    const unsigned c1 = (unsigned)(2 * H * DK + h * DK + i7);             // v channel (lanes 0..127 use it)
+    float gate_r = 0.0f, normw_r = 0.0f;                                  // the epilogue's operands
+    struct RowIn {
+        uint2 w0, w1;
+        bf16_t x0[TAPS], x1[TAPS];
+        bf16_t a_raw, b_raw, g_raw, nw_raw;
+        float dtb;
+    };
+    auto load_row = [&](int r, RowIn& in) {
         const long long gr = rr.row0 + r;
+        in.w0 = *reinterpret_cast<const uint2*>(cw + (size_t)c0 * TAPS);
+        in.w1 = *reinterpret_cast<const uint2*>(cw + (size_t)c1 * TAPS);
 #pragma unroll
-        for (int item = 0; item < 2; ++item) {
-            const bool is_conv = item == 0 || t < DK;
-            if (is_conv) {
-                const int which = item == 0 ? (t >> 7) : 2;   // 0 q, 1 k, 2 v
-                const int i = t & (DK - 1);
-                const unsigned c = (unsigned)(which * H * DK + h * DK + i);
-                const uint2 w4 = *reinterpret_cast<const uint2*>(cw + (size_t)c * TAPS);   // the 4 taps
-                const float wt[TAPS] = {__uint_as_float(w4.x << 16), __uint_as_float(w4.x & 0xffff0000u),
-                                        __uint_as_float(w4.y << 16), __uint_as_float(w4.y & 0xffff0000u)};
-                float acc = 0.0f;
-#pragma unroll
-                for (int tap = 0; tap < TAPS; ++tap) {
-                    const int at = r + tap;
-                    const bf16_t* src = at < WINDOW ? cs + (long long)at * C : P + (rr.row0 + at - WINDOW) * p_stride;
-                    acc = acc + wt[tap] * bf2f(src[c]);
-                }
-                const float act = bfround(acc / (1.0f + expf(-acc)));
-                if (which == 0) qs[i] = act;
-                else if (which == 1) ks[i] = act;
-                else vs[i] = act;
-            } else {
-                const unsigned i = (unsigned)(t - DK);
-                const float a = bf2f((A + gr * a_stride + h * DK)[i]) + (dt_bias + h * DK)[i];
-                gs[i] = expf(lower * sigmoidf_(decay_rate * a));
-            }
+        for (int tap = 0; tap < TAPS; ++tap) {
+            const int at = r + tap;
+            const bf16_t* src = at < WINDOW ? cs + (long long)at * C : P + (rr.row0 + at - WINDOW) * p_stride;
+            in.x0[tap] = src[c0];
+            in.x1[tap] = src[c1];
         }
-        if (t == THREADS - 1) beta_s = bfround(sigmoidf_(bf2f(P[gr * p_stride + b_off + h])));
+        in.a_raw = (A + gr * a_stride + h * DK)[(unsigned)i7];
+        in.dtb = (dt_bias + h * DK)[(unsigned)i7];
+        in.b_raw = P[gr * p_stride + b_off + h];
+        in.g_raw = (G + gr * g_stride + h * DV)[(unsigned)i7];
+        in.nw_raw = norm_w[i7];
+    };
+    auto prologue = [&](const RowIn& in) {
+        const uint2 w0 = in.w0, w1 = in.w1;
+        const bf16_t (&x0)[TAPS] = in.x0;
+        const bf16_t (&x1)[TAPS] = in.x1;
+        const bf16_t a_raw = in.a_raw, b_raw = in.b_raw;
+        const float dtb = in.dtb;
+        gate_r = bf2f(in.g_raw);
+        normw_r = bf2f(in.nw_raw);
+        // conv + SiLU, one bf16 rounding (cpu.rs:257-281)
+        auto conv1 = [&](const uint2 w4, const bf16_t (&x)[TAPS]) -> float {
+            const float wt[TAPS] = {__uint_as_float(w4.x << 16), __uint_as_float(w4.x & 0xffff0000u),
+                                    __uint_as_float(w4.y << 16), __uint_as_float(w4.y & 0xffff0000u)};
+            float acc = 0.0f;
+#pragma unroll
+            for (int tap = 0; tap < TAPS; ++tap) acc = acc + wt[tap] * bf2f(x[tap]);
+            return bfround(acc / (1.0f + expf(-acc)));
+        };
+        const float act0 = conv1(w0, x0);
+        if (t < DK) qs[i7] = act0; else ks[i7] = act0;
+        if (t < DK) {
+            vs[i7] = conv1(w1, x1);
+        } else {
+            gs[i7] = expf(lower * sigmoidf_(decay_rate * (bf2f(a_raw) + dtb)));   // cpu.rs:247-249
+        }
+        if (t == THREADS - 1) beta_s = bfround(sigmoidf_(bf2f(b_raw)));
         __syncthreads();
         if (wave == 0) {
-            float* x = lane < 32 ? qs : ks;    // lanes 0..31 take q, lanes 32..63 take k
+            float* x = lane < 32 ? qs : ks;    // L2 norms (cpu.rs:305-315): lanes 0..31 take q, lanes 32..63 take k
             const int l32 = lane & 31;
             float v4[4];
             const float ss = sumsq128(x, l32, v4);
@@ -132,12 +152,19 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
         __syncthreads();
     };
 
-    prologue(0);
-
+    // The state's loads go out first (measured faster than the reverse order), then the first row's inputs.
+    // Between rows the state stays in its stored form (`raw`: packed bf16 pairs, or f32 bits): a bf16 state is
+    // rounded after every row anyway, and the packed form halves the registers it holds.
+    uint4 raw[M::STEPS];
+    load_state<S>(state_in + sbase, soff_lane, raw);
     int r = 0;
     do {   // rows >= 1 here; a do-while leaves no zero-trip path that would keep the loaded state alive
         const long long gr = rr.row0 + r;
-        prologue(r);
+        {
+            RowIn in;
+            load_row(r, in);
+            prologue(in);
+        }
         const float beta = beta_s;
         float kk[KPL], qq[KPL], gg[KPL];
 #pragma unroll
@@ -177,9 +204,8 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
         __syncthreads();
         if (t < DV) {
             const float yn = ys[t] * rinv_s;
-            const float yw = bf2f(norm_w[t]) * yn;
-            const float gate = bf2f((G + gr * g_stride + h * DV)[(unsigned)t]);
-            (out + gr * out_stride + h * DV)[(unsigned)t] = f2bf(yw * sigmoidf_(gate));
+            const float yw = normw_r * yn;
+            (out + gr * out_stride + h * DV)[(unsigned)t] = f2bf(yw * sigmoidf_(gate_r));
         }
         __syncthreads();
     } while (++r < rows);
