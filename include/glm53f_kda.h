@@ -197,7 +197,7 @@ int glm53f_kda_conv_shift_batch(int32_t channels, int32_t layers, int32_t batch,
 
 /**
  * Bytes of workspace for the prefill to run `rows_per_pass` rows of every request per pass; 0 on bad
- * arguments. On this build a chunk is 64 rows and costs 75,264 bytes per head and request. Replaces
+ * arguments. On this build a chunk is 64 rows and costs 74,240 bytes per head and request. Replaces
  * glm53f_kda_prefill_workspace_bytes (header :204, kda_prefill.cu:695-698; 34,816 bytes per 16 rows there).
  */
 int64_t glm53f_kda_prefill_workspace_bytes(int32_t heads, int32_t batch, int32_t rows_per_pass);
@@ -242,9 +242,9 @@ int glm53f_kda_prefill_batch(int32_t heads, int32_t batch, const int32_t* cu_row
                              float* workspace, int64_t workspace_bytes, glm53f_stream_t stream);
 
 /**
- * glm53f_kda_prefill_batch with bf16 states in the pool. The state is carried in f32 on chip across all
- * chunks of a pass and rounded to bf16 when a pass stores it (passes are whole chunks counted from each
- * request's first row). Replaces glm53f_kda_prefill_batch_bf16state (header :260-270,
+ * glm53f_kda_prefill_batch with bf16 states in the pool. The state is carried in f32 accumulators across a
+ * chunk of 64 rows and rounded to bf16 at the end of every chunk (chunks count from each request's first row),
+ * so the results still do not depend on the workspace size. Replaces glm53f_kda_prefill_batch_bf16state (header :260-270,
  * kda_prefill.cu:727-742).
  */
 int glm53f_kda_prefill_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,

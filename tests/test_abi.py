@@ -1,0 +1,44 @@
+"""The C ABI as a boundary: the built library loads and exports every symbol include/glm53f_kda.h declares, the
+header keeps the reference's 13 entry points (crates/glm53f-kda/tests/provenance.rs:41-69), and the ctypes
+prototypes agree with the header's parameter counts. No compute call: runs without a GPU."""
+import os
+import re
+
+from glm53f_kda import ffi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declarations():
+    text = open(os.path.join(ROOT, "include", "glm53f_kda.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for m in re.finditer(r"\b(?:int|int64_t|const char\*)\s+(glm53f_kda_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        args = m.group(2).strip()
+        out[m.group(1)] = 0 if args in ("", "void") else len(args.split(","))
+    return out
+
+
+def test_header_declares_the_reference_entry_points():
+    decl = declarations()
+    for name in ffi.REFERENCE_SYMBOLS:
+        assert name in decl, name
+    assert len(ffi.REFERENCE_SYMBOLS) == 13
+    extra = set(decl) - set(ffi.REFERENCE_SYMBOLS)
+    assert extra == {"glm53f_kda_verify_batch_bf16state", "glm53f_kda_select_batch_bf16state", "glm53f_kda_arch"}
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ffi.lib()
+    decl = declarations()
+    assert set(decl) == set(ffi.PROTOTYPES)
+    for name, nargs in decl.items():
+        assert hasattr(lib, name), name
+        assert len(ffi.PROTOTYPES[name][1]) == nargs, name
+    assert lib.glm53f_kda_arch() == b"gfx950"
+
+
+def test_workspace_bytes_is_a_pure_host_function():
+    assert ffi.glm53f_kda_prefill_workspace_bytes(64, 1, 2048) == 32 * 74240 * 64
+    assert ffi.glm53f_kda_prefill_workspace_bytes(64, 1, 1) == 74240 * 64
+    assert ffi.glm53f_kda_prefill_workspace_bytes(0, 1, 16) == 0
