@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the KDA hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|copy]
 
 Prints ONE JSON line. The headline `value` is the decode step's state traffic in GB/s at BASELINE config 1
 (16 slots x 1 token out of a 48-slot bf16 pool, 64 heads, 34 layers each with its own pool so the working set
@@ -293,12 +293,24 @@ def bench_verify(steps, warmup, stream):
 
 # ------------------------------------------------------------------------------------------------ main
 
+# ------------------------------------------------------------------------------------------------ copy
+
+def bench_copy(steps, warmup, stream):
+    """A plain device-to-device copy of known size: the yardstick that FETCH_SIZE / WRITE_SIZE counter readings
+    of the kernels above are scaled by, and the copy bandwidth this box reaches."""
+    n = 1 << 29                                          # 512 Mi bf16 elements = 1 GiB read + 1 GiB written
+    src = torch.ones(n, dtype=torch.bfloat16, device=DEV)
+    dst = torch.empty_like(src)
+    ms = timed(lambda: dst.copy_(src), steps, warmup, stream)
+    return {"bytes_read": 2 * n, "bytes_written": 2 * n, "ms": ms, "GBps": 4 * n / (ms * 1e-3) / 1e9}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", choices=["decode", "prefill", "verify"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "verify", "copy"], default=None)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -336,6 +348,10 @@ def main():
         if args.only == "verify":
             line.update({"value": ver["roofline"]["achieved"], "ms_per_step": ver["verify_ms_per_layer"],
                          "roofline": ver["roofline"], "config": ver["config"]})
+    if args.only == "copy":
+        cp = bench_copy(args.steps, args.warmup, stream)
+        line.update({"copy": cp, "value": cp["GBps"], "ms_per_step": cp["ms"],
+                     "config": {"workload": "1 GiB device-to-device copy (counter yardstick)"}})
     print(json.dumps(line))
 
 
