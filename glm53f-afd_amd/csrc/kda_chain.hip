@@ -100,14 +100,14 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
 #pragma unroll
         for (int tap = 0; tap < TAPS; ++tap) {
             const int at = r + tap;
-            const bf16_t* src = at < WINDOW ? cs + (long long)at * C : P + (rr.row0 + at - WINDOW) * p_stride;
+            const bf16_t* src = uniform_ptr(at < WINDOW ? cs + (long long)at * C : P + (rr.row0 + at - WINDOW) * p_stride);
             in.x0[tap] = src[c0];
             in.x1[tap] = src[c1];
         }
-        in.a_raw = (A + gr * a_stride + h * DK)[(unsigned)i7];
+        in.a_raw = uniform_ptr(A + gr * a_stride + h * DK)[(unsigned)i7];
         in.dtb = (dt_bias + h * DK)[(unsigned)i7];
-        in.b_raw = P[gr * p_stride + b_off + h];
-        in.g_raw = (G + gr * g_stride + h * DV)[(unsigned)i7];
+        in.b_raw = *uniform_ptr(P + gr * p_stride + b_off + h);
+        in.g_raw = uniform_ptr(G + gr * g_stride + h * DV)[(unsigned)i7];
         in.nw_raw = norm_w[i7];
     };
     auto prologue = [&](const RowIn& in) {
@@ -183,14 +183,14 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
             if (lane % M::LPR == 0) ys[row] = bfround(o);
             raw[j] = pack<S>(s);        // rounds a bf16 state (after the row's read-out)
         }
-        if (ckpt != nullptr) store_raw<S>(ckpt + (gr * H + h) * (long long)(DV * DK), soff_lane, raw);
+        if (ckpt != nullptr) store_raw<S>(uniform_ptr(ckpt + (gr * H + h) * (long long)(DV * DK)), soff_lane, raw);
         if (k_save != nullptr) {
             const long long base = (gr * H + h) * DK;
             if (t < DK) {
-                (k_save + base)[(unsigned)t] = ks[t];
-                (g_save + base)[(unsigned)t] = gs[t];
+                uniform_ptr(k_save + base)[(unsigned)t] = ks[t];
+                uniform_ptr(g_save + base)[(unsigned)t] = gs[t];
             } else {
-                (v_save + base)[(unsigned)(t - DK)] = f2bf(vs[t - DK]);
+                uniform_ptr(v_save + base)[(unsigned)(t - DK)] = f2bf(vs[t - DK]);
             }
             if (t == 0) b_save[gr * H + h] = beta;
         }
@@ -205,7 +205,7 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
         if (t < DV) {
             const float yn = ys[t] * rinv_s;
             const float yw = normw_r * yn;
-            (out + gr * out_stride + h * DV)[(unsigned)t] = f2bf(yw * sigmoidf_(gate_r));
+            uniform_ptr(out + gr * out_stride + h * DV)[(unsigned)t] = f2bf(yw * sigmoidf_(gate_r));
         }
         __syncthreads();
     } while (++r < rows);

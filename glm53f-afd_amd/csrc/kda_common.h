@@ -33,6 +33,16 @@ __device__ __forceinline__ float bfround(float x) { return bf2f(f2bf(x)); }
 
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
 
+// A wave-uniform pointer forced into scalar registers and made opaque to loop strength reduction: addressing
+// through it is "scalar base + 32-bit lane offset", and no per-lane 64-bit pointer is carried across a loop.
+template <typename T>
+__device__ __forceinline__ T* uniform_ptr(T* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
+}
+
 // Request b's global rows: [row0, row0 + rows). Without cu_rows: one request of rows1 rows.
 struct RowRange {
     long long row0;
