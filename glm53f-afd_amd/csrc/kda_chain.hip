@@ -152,20 +152,30 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
         __syncthreads();
     };
 
-    // The state's loads go out first (measured faster than the reverse order), then the first row's inputs.
-    // Between rows the state stays in its stored form (`raw`: packed bf16 pairs, or f32 bits): a bf16 state is
-    // rounded after every row anyway, and the packed form halves the registers it holds.
+    // The first row's inputs are requested before the state (the scheduling barriers keep that order), so the
+    // prologue waits for them alone and runs while the state streams in. Between rows the state stays in its
+    // stored form (`raw`: packed bf16 pairs, or f32 bits): a bf16 state is rounded after every row anyway, and
+    // the packed form halves the registers it holds. With a bf16 state there are registers to spare, and the
+    // next row's inputs are requested before this row's update; an f32 state requests them after the epilogue.
+    constexpr bool kPrefetch = M::kRound;
     uint4 raw[M::STEPS];
+    RowIn in;
+    load_row(0, in);
+    __builtin_amdgcn_sched_barrier(0);
     load_state<S>(state_in + sbase, soff_lane, raw);
+    __builtin_amdgcn_sched_barrier(0);
     int r = 0;
     do {   // rows >= 1 here; a do-while leaves no zero-trip path that would keep the loaded state alive
         const long long gr = rr.row0 + r;
-        {
-            RowIn in;
-            load_row(r, in);
-            prologue(in);
+        prologue(in);
+        if constexpr (kPrefetch) {
+            if (r + 1 < rows) load_row(r + 1, in);
         }
         const float beta = beta_s;
+        // Stores leave as soon as a step's 16 or 8 value rows are final, so they overlap the remaining steps
+        // and the row's epilogue: the checkpoint of every row, and the state itself in the last row.
+        S* const ck_row = ckpt != nullptr ? uniform_ptr(ckpt + (gr * H + h) * (long long)(DV * DK)) : nullptr;
+        S* const st_row = (state_out != nullptr && r + 1 == rows) ? uniform_ptr(state_out + sbase) : nullptr;
         float kk[KPL], qq[KPL], gg[KPL];
 #pragma unroll
         for (int c = 0; c < KPL; ++c) {
@@ -182,8 +192,9 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
             const float o = read_row<S>(s, qq);
             if (lane % M::LPR == 0) ys[row] = bfround(o);
             raw[j] = pack<S>(s);        // rounds a bf16 state (after the row's read-out)
+            if (ck_row != nullptr) st128((ck_row + j * M::RPS * DK) + soff_lane, raw[j]);
+            if (st_row != nullptr) st128((st_row + j * M::RPS * DK) + soff_lane, raw[j]);
         }
-        if (ckpt != nullptr) store_raw<S>(uniform_ptr(ckpt + (gr * H + h) * (long long)(DV * DK)), soff_lane, raw);
         if (k_save != nullptr) {
             const long long base = (gr * H + h) * DK;
             if (t < DK) {
@@ -208,8 +219,10 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
             uniform_ptr(out + gr * out_stride + h * DV)[(unsigned)t] = f2bf(yw * sigmoidf_(gate_r));
         }
         __syncthreads();
+        if constexpr (!kPrefetch) {
+            if (r + 1 < rows) load_row(r + 1, in);
+        }
     } while (++r < rows);
-    if (state_out != nullptr) store_raw<S>(state_out + sbase, soff_lane, raw);
 }
 
 // Replay of saved rows (reference: kda.cu:214-253, cpu.rs:486-508): workgroup (layer * H + h, b). Waves are

@@ -40,7 +40,10 @@ __device__ __forceinline__ T* uniform_ptr(T* p) {
     const uint64_t v = reinterpret_cast<uint64_t>(p);
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
     const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
+    // Through a global-address-space pointer, so that accesses stay global_* instructions (a pointer made
+    // from an integer would otherwise be generic and use flat_* ones, which wait on both memory counters).
+    typedef __attribute__((address_space(1))) T* global_ptr_t;
+    return (T*)reinterpret_cast<global_ptr_t>(((uint64_t)hi << 32) | lo);
 }
 
 // Request b's global rows: [row0, row0 + rows). Without cu_rows: one request of rows1 rows.

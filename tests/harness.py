@@ -255,6 +255,14 @@ def ulps(a, b):
     return int(d.max()) if d.size else 0, int((d > 0).sum())
 
 
+def bf16_steps(a, b):
+    """How many representable bf16 values apart two arrays of bf16-valued floats are."""
+    def key(x):
+        u = np.asarray(x, np.float32).view(np.uint32).astype(np.int64) >> 16
+        return np.where(u & 0x8000, -(u & 0x7FFF), u)
+    return np.abs(key(a) - key(b))
+
+
 def bits(x):
     return np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
 

@@ -123,5 +123,8 @@ def test_gpu_prefill_meets_the_vectors(vec):
     p, conv, s0, rows = case(vec, "prefill")
     out, state, conv_after = hs.prefill_gpu(p, conv, s0, rows)
     assert hs.rel_err(state, vec["prefill.state_out"]) <= 1e-3
-    assert hs.max_abs(out, vec["prefill.out"]) <= 2e-2
+    # 2e-2, or two representable bf16 values where those are further apart than that (outputs beyond 2): the
+    # read-out and the gated norm each round to bf16, so a last-place difference can move an output two steps.
+    far = np.abs(out - vec["prefill.out"]) > 2e-2
+    assert not far.any() or hs.bf16_steps(out, vec["prefill.out"])[far].max() <= 2
     assert same_bits(conv_after, vec["prefill.conv_after"])

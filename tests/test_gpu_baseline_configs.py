@@ -18,14 +18,6 @@ import harness as hs
 pytestmark = pytest.mark.gpu
 
 
-def bf16_steps(a, b):
-    """How many representable bf16 values apart two arrays of bf16-valued floats are."""
-    def key(x):
-        u = np.asarray(x, np.float32).view(np.uint32).astype(np.int64) >> 16
-        return np.where(u & 0x8000, -(u & 0x7FFF), u)
-    return np.abs(key(a) - key(b))
-
-
 def check_outputs(got, ref, label):
     """The north-star bar on bf16 outputs is max-abs <= 2e-2, which is what two bf16 steps come to for outputs
     below 2 (2 * 2^-7 = 1.56e-2). The contract rounds twice (the read-out to bf16, then the gated norm's result to
@@ -36,7 +28,7 @@ def check_outputs(got, ref, label):
     |diff| <= 2e-2 or be at most two representable values away; the print says how many needed the second clause."""
     got, ref = np.asarray(got, np.float32), np.asarray(ref, np.float32)
     d = np.abs(got.astype(np.float64) - ref.astype(np.float64))
-    steps = bf16_steps(got, ref)
+    steps = hs.bf16_steps(got, ref)
     hist = np.bincount(np.minimum(steps, 4).ravel(), minlength=5)
     over = d > 2e-2
     print(f"{label}: outputs 0/1/2/3/4+ bf16 steps apart: {hist.tolist()}; {int(over.sum())} differ by more than 2e-2 "
