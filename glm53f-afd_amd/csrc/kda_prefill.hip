@@ -595,7 +595,10 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         const S* state_in, S* state_out, const long long* __restrict__ state_off,
         bf16_t* __restrict__ out, long long out_stride, const unsigned char* __restrict__ ws) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const int h = blockIdx.x / VBLOCKS, vb = blockIdx.x % VBLOCKS, b = blockIdx.y;
+    // Workgroups go to the eight XCDs round robin by their linear index. The value-column blocks of one head
+    // read the same W, Qg, Kg and M, so they are spaced H apart (a multiple of 8 for the model's 64 heads):
+    // they run on one XCD and share its L2 instead of fetching the workspace once per block.
+    const int h = blockIdx.x % H, vb = blockIdx.x / H, b = blockIdx.y;
     const RowRange rr = request_rows(cu_rows, b, rows1);
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
     const int left = rr.rows - sub0;                              // rows of this request from this pass on
