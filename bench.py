@@ -3,14 +3,14 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|copy]
 
-Prints ONE JSON line. The headline `value` is the decode step's state traffic in GB/s at BASELINE config 1
+Prints ONE JSON line. The headline `value` is the decode step's state traffic in GB/s in the 16-slot decode configuration
 (16 slots x 1 token out of a 48-slot bf16 pool, 64 heads, 34 layers each with its own pool so the working set
 exceeds the last-level cache); a "step" is one decode step over the 34 KDA layers (chain + conv shift per
-layer). The same line carries the chunked prefill (config 2: T = 8192 as four sequential 2048-row calls on one
-slot) and the checkpointing verify (config 4: 48 slots x 16 drafts) under `prefill` and `verify`, each with its
+layer). The same line carries the chunked prefill (T = 8192 as four sequential 2048-row calls on one
+slot) and the checkpointing verify (48 slots x 16 drafts) under `prefill` and `verify`, each with its
 own roofline object, and the CPU oracle timed on this host's cores as `cpu_baseline`.
 
-Inputs are synthetic with BASELINE's distributions, generated on the GPU; all buffers are resident in HBM
+Inputs are synthetic with the distributions of the benchmark definition, generated on the GPU; all buffers are resident in HBM
 before the timed region. Kernel durations are measured with events on the stream the kernels are launched on.
 """
 import argparse
@@ -29,6 +29,14 @@ import torch
 
 from glm53f_kda import DK, DV, HEADS, LAYERS, WINDOW, channels, ffi, state_len
 
+# HBM bytes per launch from the FETCH_SIZE and WRITE_SIZE counters (one rocprofv3 --pmc run each over this
+# script's legs, scaled by the same counters over the 1 GiB copy of --only copy: x2.00 and x1.00). Measured
+# offline; the summaries are kept in profiles/.
+TRAFFIC_BYTES = {
+    "decode_chain": (36_792 + 33_024) * 1024,            # per chain launch, 16 slots x 1 row
+    "verify_chain": (223_800 + 1_585_152) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
+    "prefill_2048_rows": (139_573 + 149_043 + 152_661 + 36_864 + 65_580 + 32_768 + 172 + 144) * 1024,
+}
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
 DEV = "cuda:0"
@@ -41,7 +49,7 @@ def ptr(t, off=0):
 
 
 class Layer:
-    """Random-init weights of one KDA layer with BASELINE's gate mapping: A_log = 0, dt_bias = 0, so
+    """Random-init weights of one KDA layer with the gate mapping of the benchmark definition: A_log = 0, dt_bias = 0, so
     g = -5 * sigmoid(a) and a = logit(softplus(z) / 5) gives g = -softplus(z)."""
 
     def __init__(self, heads, gen):
@@ -156,7 +164,8 @@ def bench_decode(steps, warmup, stream, cpu=True):
         "ms_per_step": ms_step,
         "state_GBps": layers * state_bytes / (ms_step * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "achieved": state_bytes / (ms_chain * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": state_bytes / (ms_chain * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "unit": "GB/s", "frac": state_bytes / (ms_chain * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": TRAFFIC_BYTES["decode_chain"],
                      "kernel": "chain_kernel<bf16>", "bytes_per_launch": state_bytes,
                      "us_per_launch": ms_chain * 1e3},
     }
@@ -190,7 +199,7 @@ def bench_decode(steps, warmup, stream, cpu=True):
 # ------------------------------------------------------------------------------------------------ prefill
 
 def bench_prefill(steps, warmup, stream, cpu=True):
-    """BASELINE config 2: one prompt of 8192 rows as four sequential calls of 2048 rows on one slot (the
+    """benchmark configuration 2: one prompt of 8192 rows as four sequential calls of 2048 rows on one slot (the
     engine's lanes), 64 heads, f32 carried state, conv and output gate included."""
     heads, total, lane_rows = HEADS, 8192, 2048
     gen = torch.Generator(device=DEV).manual_seed(3)
@@ -216,11 +225,12 @@ def bench_prefill(steps, warmup, stream, cpu=True):
     res = {
         "tok_per_s_per_layer": total / (ms * 1e-3), "ms_per_8192_tokens": ms,
         "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": TRAFFIC_BYTES["prefill_2048_rows"], "traffic_unit": "B per 2048-row call (4 kernels)",
                      "kernel": "prefill (intra + inter + norm + conv advance, whole call)",
                      "flops_per_token": 11_709_099, "hbm_GBps_compulsory": io_bytes / (ms * 1e-3) / 1e9,
                      "hbm_frac": io_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
-        "config": {"workload": "BASELINE config 2: T=8192 as 4 calls of 2048 rows on one slot, H=64, chunk 64, "
+        "config": {"workload": "benchmark configuration 2: T=8192 as 4 calls of 2048 rows on one slot, H=64, chunk 64, "
                                "bf16 rows, f32 state, conv + output gate", "workspace_MB": ws_bytes / 1e6},
     }
     if cpu:
@@ -244,7 +254,7 @@ def bench_prefill(steps, warmup, stream, cpu=True):
 # ------------------------------------------------------------------------------------------------ verify
 
 def bench_verify(steps, warmup, stream):
-    """BASELINE config 4: 48 slots x 16 draft rows, bf16 state, a checkpoint after every row, then the commit by
+    """benchmark configuration 4: 48 slots x 16 draft rows, bf16 state, a checkpoint after every row, then the commit by
     selection with an accepted length per slot drawn uniformly from [0, 16]."""
     heads, slots_n, drafts, layers = HEADS, 48, 16, 2
     gen = torch.Generator(device=DEV).manual_seed(4)
@@ -283,10 +293,10 @@ def bench_verify(steps, warmup, stream):
     return {
         "verify_ms_per_layer": ms_v, "select_ms_per_layer": ms_s,
         "roofline": {"bound": "hbm", "achieved": vbytes / (ms_v * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": vbytes / (ms_v * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": vbytes / (ms_v * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": TRAFFIC_BYTES["verify_chain"],
                      "kernel": "chain_kernel<bf16> with checkpoints", "bytes_per_launch": vbytes},
         "select_GBps": sbytes / (ms_s * 1e-3) / 1e9,
-        "config": {"workload": "BASELINE config 4: verify 48 slots x 16 drafts, bf16 state, per-row checkpoints; "
+        "config": {"workload": "benchmark configuration 4: verify 48 slots x 16 drafts, bf16 state, per-row checkpoints; "
                                "select with keep ~ U{0..16}", "kept_slots": kept},
     }
 
@@ -324,13 +334,13 @@ def main():
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream()
     line = {"metric": METRIC, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32 (bf16 state and rows)",
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
             "data": "synthetic"}
     dec = None
     if args.only in (None, "decode"):
         dec = bench_decode(args.steps, args.warmup, stream, cpu=not args.no_cpu)
         line.update({"value": dec["state_GBps"], "ms_per_step": dec["ms_per_step"], "roofline": dec["roofline"],
-                     "config": {"workload": "BASELINE config 1: decode, 16 slots x 1 token of a 48-slot bf16 pool, "
+                     "config": {"workload": "configs[1]: decode, 16 slots x 1 token of a 48-slot bf16 pool, "
                                             "H=64, dk=dv=128, 34 layers (one pool each), chain + conv shift per layer",
                                 "slots": 16, "pool_slots": 48, "heads": 64, "layers": 34}})
         if "cpu_baseline" in dec:

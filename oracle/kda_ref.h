@@ -58,7 +58,7 @@ float kda_rng_uniform(kda_rng* r, float lo, float hi);
 float kda_rng_uniform_bf16(kda_rng* r, float lo, float hi);
 void kda_rng_fill(kda_rng* r, float* out, int64_t n, float lo, float hi);
 void kda_rng_fill_bf16(kda_rng* r, float* out, int64_t n, float lo, float hi);
-/* Standard normal by Box-Muller on two 24-bit uniforms (not in the reference: BASELINE's distributions). */
+/* Standard normal by Box-Muller on two 24-bit uniforms (not in the reference: the benchmark definition's distributions). */
 float kda_rng_normal(kda_rng* r);
 void kda_rng_fill_normal(kda_rng* r, float* out, int64_t n);
 

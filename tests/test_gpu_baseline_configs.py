@@ -1,4 +1,4 @@
-"""BASELINE's configurations at their stated sizes, through the C ABI.
+"""The benchmark definition's configurations at their stated sizes, through the C ABI.
 
 Config 1 (decode, 16 of 48 slots) lives in test_gpu_chain.py. Here: config 2 (T = 8192 as four 2048-row calls)
 against the FP32 recurrent oracle with the north-star tolerances; config 3 (varlen packed prefill) at a size the

@@ -297,7 +297,7 @@ def test_verify_checkpoints_and_select_are_bit_exact():
 
 
 def test_baseline_config1_decode_16_of_48_slots():
-    """BASELINE config 1: 16 slots x 1 token from a 48-slot bf16 pool, H=64; q,k,v ~ N(0,1) before the conv,
+    """benchmark configuration 1: 16 slots x 1 token from a 48-slot bf16 pool, H=64; q,k,v ~ N(0,1) before the conv,
     beta = sigmoid(N(0,1)), g = -softplus(N(0,1)) (through A_log = dt_bias = 0 and a = logit(softplus(z)/5)),
     initial states ~ N(0, 0.02), random slot ids without repeats."""
     heads, slots_n, batch = 64, 48, 16

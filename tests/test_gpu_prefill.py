@@ -19,14 +19,14 @@ pytestmark = pytest.mark.gpu
 
 STATE_TOL = 1e-3          # max |diff| / max |ref| against the FP32 recurrent reference
 OUT_REL = 2.0 ** -7       # bf16 outputs, normwise: the reference's own bound (gpu_prefill.rs:245-247)
-OUT_ABS = 2e-2            # bf16 outputs, max-abs, on BASELINE's distributions (outputs of order one)
+OUT_ABS = 2e-2            # bf16 outputs, max-abs, on the benchmark definition's distributions (outputs of order one)
 FLIP_FRACTION = 0.25      # at most this share of outputs may differ at all
 
 
 def out_ok(got, ref):
     """Normwise 2^-7 against the largest output. With the reference's synthetic ranges (norm weights up to 1.75,
     gates up to sigmoid(4)) outputs reach 7, where one bf16 ulp is 2^-5: a max-abs bound of 2e-2 cannot hold for
-    any kernel that is not bit-exact, so that bound is asserted on BASELINE's distributions instead
+    any kernel that is not bit-exact, so that bound is asserted on the benchmark definition's distributions instead
     (test_baseline_config2_*)."""
     return hs.rel_err(got, ref) <= OUT_REL
 

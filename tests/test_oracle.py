@@ -424,7 +424,7 @@ def test_chunked_head_against_f64_textbook():
 
 
 def test_baseline_config0_chunked_vs_recurrent():
-    """BASELINE config 0: one sequence, T=256, 64 heads, chunk 64, fp32, zero initial state."""
+    """benchmark configuration 0: one sequence, T=256, 64 heads, chunk 64, fp32, zero initial state."""
     heads, t = 64, 256
     rng = o.Rng(2026)
     q = rng.normal(t * heads * DK)
