@@ -12,7 +12,8 @@
 //     (15 rows at the -5.8 bound), so these operands are bf16 split into hi + lo (three products);
 //   * between sub-chunks around a row in between (the end of a sub-chunk, or the middle of the chunk), where
 //     both exponents are <= 0 and the operands are fp16 (11-bit mantissa at the bf16 MFMA rate).
-// Everything that feeds the state is fp16 or split bf16; T is inverted in f32.
+// Everything that feeds the state is fp16 or split bf16. Only the diagonal 16x16 blocks of T are formed (in f32);
+// W and U come from a block forward substitution on [k e^G | v] with MFMA tiles (see intra_kernel).
 //
 // Kernels per pass: intra_kernel (one workgroup per chunk, head, request: prologue + L, M, T, W, U, Qg, Kg into
 // the workspace), inter_kernel (one workgroup per head, value-column block, request: the state in MFMA
@@ -45,7 +46,7 @@ constexpr int WS_BYTES = 74240;
 
 // LDS row strides in 16-bit elements: 128- and 64-wide operand rows padded by 16 bytes, so that the sixteen
 // rows one MFMA fragment read touches fall into distinct banks.
-constexpr int LD128 = 136, LD64 = 72, LDF = 68;   // LDF: f32 [64][68]
+constexpr int LD128 = 136, LD64 = 72;
 
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
@@ -101,8 +102,10 @@ constexpr int I_BETA = I_TOT + 4 * DK * 4;        // f32 [64]
 constexpr int I_INV = I_BETA + CH * 4;            // f32 [2][64]: 1/|q| * 128^-0.5, 1/|k|
 constexpr int I_KET = I_INV + 2 * CH * 4;         // fp16 [128 keys][LD64]: k e^G, transposed
 constexpr int I_VT = I_KET + DK * LD64 * 2;       // fp16 [128 values][LD64]: v, transposed
-constexpr int I_L = I_VT + DV * LD64 * 2;         // f32 [64][LDF]: L
-constexpr int I_KC1 = I_L + CH * LDF * 4;         // fp16 [32][LD128]: column side around the chunk's middle
+constexpr int I_LN = I_VT + DV * LD64 * 2;        // fp16 [64][LD64]: -L below the block diagonal, zero elsewhere
+constexpr int LDD = SUB + 1;                      // f32 rows of a diagonal block of L
+constexpr int I_LD = I_LN + CH * LD64 * 2;        // f32 [4][16][LDD]: the diagonal blocks of L
+constexpr int I_KC1 = I_LD + 4 * SUB * LDD * 4;   // fp16 [32][LD128]: column side around the chunk's middle
 constexpr int I_PASS = I_KC1 + 32 * LD128 * 2;    // the rest is reused by every half
 constexpr int P_ROWS32 = 32 * LD128 * 2;          // one [32][LD128] 16-bit array
 constexpr int P_ROWS16 = 16 * LD128 * 2;
@@ -112,10 +115,10 @@ constexpr int I_RAWK = I_PASS + P_ROWS32;
 constexpr int I_R2 = I_DIAG + 6 * P_ROWS32;       // KR2, QR2, KC2: three [16][LD128] fp16 arrays
 constexpr int I_R1 = I_R2 + 3 * P_ROWS16;         // KR1, QR1: two [32][LD128] fp16 arrays
 constexpr int I_END = I_R1 + 2 * P_ROWS32;
-// After the halves: the inverse.
-constexpr int I_T = I_PASS;                       // f32 [64][LDF]
-constexpr int I_X = I_T + CH * LDF * 4;           // f32 [64][LDF]
-constexpr int I_TQ = I_X + CH * LDF * 4;          // fp16 [64][LD64]: T diag(beta)
+// After the halves: the block solve.
+constexpr int LDT = 40, LDZ = 24;                 // 16-bit row strides of the two arrays below (16-byte multiples)
+constexpr int I_TT = I_PASS;                      // fp16 [64][LDT]: row 16 a + i holds [T_aa diag(beta) | T_aa][i][0..32)
+constexpr int I_Z = I_TT + CH * LDT * 2;          // fp16 [16 column tiles][16][LDZ]: a tile of Z on its way back in
 // Input staging (before the operands of a half land): the half's 35 rows of q | k | v, and the chunk's gate rows.
 constexpr int LDX = DK + 8;                       // staged input rows, 16-bit elements
 constexpr int XROWS = 32 + WINDOW;
@@ -123,7 +126,7 @@ constexpr int I_XIN = I_R2;                       // bf16 [3][35][LDX]
 constexpr int I_AIN = I_PASS;                     // bf16 [64][LDX]
 static_assert(I_XIN + 3 * XROWS * LDX * 2 <= I_END, "input staging must fit behind the diagonal operands");
 constexpr int INTRA_LDS = I_END;
-static_assert(I_TQ + CH * LD64 * 2 <= I_END, "inverse scratch must fit the per-half region");
+static_assert(I_Z + 16 * SUB * LDZ * 2 <= I_END, "solve scratch must fit the per-half region");
 static_assert(INTRA_LDS <= 160 * 1024, "intra_kernel LDS");
 
 // NROWS rows of 128 bf16 on their way from global memory to LDS rows of LDX elements. src(row) is the row's
@@ -190,7 +193,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
     float* inv_s = reinterpret_cast<float*>(smem + I_INV);
     uint16_t* keT = reinterpret_cast<uint16_t*>(smem + I_KET);
     uint16_t* VT = reinterpret_cast<uint16_t*>(smem + I_VT);
-    float* Ls = reinterpret_cast<float*>(smem + I_L);
+    uint16_t* Ln = reinterpret_cast<uint16_t*>(smem + I_LN);
+    float* Ld = reinterpret_cast<float*>(smem + I_LD);
     uint16_t* KC1 = reinterpret_cast<uint16_t*>(smem + I_KC1);
 
     // ---- gates of the whole chunk: cumulative log decay of this lane's channel inside its two sub-chunks
@@ -422,13 +426,20 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
             const uint16_t* QR1 = KR1 + 32 * LD128;
             uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
             const int rl = 4 * (lane >> 4), cl = lane & 15;   // this lane's rows rl..rl+3 and column cl of a tile
-            // Store a finished tile at block (rb, cb): L = beta_i * acc (strictly lower on the diagonal) to LDS,
-            // M (lower with the diagonal) to the workspace.
+            // Store a finished tile at block (rb, cb). L = beta_i * acc: a diagonal block (strictly lower) in f32 for
+            // the inversion, a block below the diagonal negated in fp16 as an MFMA operand of the block solve.
+            // M (lower with the diagonal) goes to the workspace.
             auto put_L = [&](f32x4 acc, int rb, int cb) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const int gi = SUB * rb + rl + r, gj = SUB * cb + cl;
-                    Ls[gi * LDF + gj] = (rb != cb || gj < gi) ? beta_s[gi] * acc[r] : 0.0f;
+                    const int li = rl + r, gi = SUB * rb + li, gj = SUB * cb + cl;
+                    const float v = beta_s[gi] * acc[r];
+                    if (rb == cb) {
+                        Ld[(SUB * rb + li) * LDD + cl] = cl < li ? v : 0.0f;
+                        Ln[gi * LD64 + gj] = 0;
+                    } else {
+                        Ln[gi * LD64 + gj] = f2h(-v);
+                    }
                 }
             };
             auto put_M = [&](f32x4 acc, int rb, int cb) {
@@ -461,7 +472,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         }
         __syncthreads();
     }
-    // M above the block diagonal is zero: blocks (0,1), (0,2), (0,3), (1,2), (1,3), (2,3)
+    // M and -L above the block diagonal are zero: blocks (0,1), (0,2), (0,3), (1,2), (1,3), (2,3)
     {
         uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
         for (int e = t; e < 6 * 256; e += THREADS) {
@@ -469,84 +480,90 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
             const int rb = blk < 3 ? 0 : (blk < 5 ? 1 : 2);
             const int cb = blk < 3 ? blk + 1 : (blk < 5 ? blk - 1 : 3);
             Mg[(SUB * rb + r) * CH + SUB * cb + cc] = 0;
+            Ln[(SUB * rb + r) * LD64 + SUB * cb + cc] = 0;
         }
     }
 
-    // ---- T = (I + L)^-1 in f32
-    float* Ts = reinterpret_cast<float*>(smem + I_T);
-    float* Xs = reinterpret_cast<float*>(smem + I_X);
-    uint16_t* Tq = reinterpret_cast<uint16_t*>(smem + I_TQ);
+    // ---- the diagonal blocks of T = (I + L)^-1 in f32 by forward substitution: lane (a, j) solves column j of
+    // block a and leaves it as fp16 operands, scaled by beta_j (T' = T diag(beta)) and plain.
+    uint16_t* TT = reinterpret_cast<uint16_t*>(smem + I_TT);
     if (t < CH) {
-        // diagonal blocks by forward substitution: lane (a, j) solves column j of block a
         const int a = t >> 4, j = t & 15;
+        const float bj = beta_s[t];
         float x[SUB];
 #pragma unroll
         for (int i = 0; i < SUB; ++i) {
             float acc = 0.0f;
 #pragma unroll
-            for (int m = 0; m < i; ++m) acc = __builtin_fmaf(Ls[(SUB * a + i) * LDF + SUB * a + m], x[m], acc);
+            for (int m = 0; m < i; ++m) acc = __builtin_fmaf(Ld[(SUB * a + i) * LDD + m], x[m], acc);
             x[i] = i < j ? 0.0f : (i == j ? 1.0f : -acc);
-            Ts[(SUB * a + i) * LDF + SUB * a + j] = x[i];
+            TT[(SUB * a + i) * LDT + j] = f2h(x[i] * bj);
+            TT[(SUB * a + i) * LDT + SUB + j] = f2h(x[i]);
         }
-    }
-    __syncthreads();
-    // off-diagonal blocks by distance from the diagonal: T_ab = -T_aa sum_{c=b}^{a-1} L_ac T_cb
-    {
-        const int ei = t >> 4, ej = t & 15;       // this lane's element of a 16x16 block
-#pragma unroll 1
-        for (int dist = 1; dist < 4; ++dist) {
-            for (int bb = 0; bb + dist < 4; ++bb) {
-                const int a = bb + dist;
-                float acc = 0.0f;
-                for (int cc = bb; cc < a; ++cc)
-#pragma unroll
-                    for (int m = 0; m < SUB; ++m)
-                        acc = __builtin_fmaf(Ls[(SUB * a + ei) * LDF + SUB * cc + m], Ts[(SUB * cc + m) * LDF + SUB * bb + ej], acc);
-                Xs[(SUB * a + ei) * LDF + SUB * bb + ej] = acc;
-            }
-            __syncthreads();
-            for (int bb = 0; bb + dist < 4; ++bb) {
-                const int a = bb + dist;
-                float acc = 0.0f;
-#pragma unroll
-                for (int m = 0; m < SUB; ++m)
-                    acc = __builtin_fmaf(Ts[(SUB * a + ei) * LDF + SUB * a + m], Xs[(SUB * a + m) * LDF + SUB * bb + ej], acc);
-                Ts[(SUB * a + ei) * LDF + SUB * bb + ej] = -acc;
-            }
-            __syncthreads();
-        }
-    }
-    // T' = T diag(beta) as an fp16 operand (zero above the diagonal)
-    for (int e = t; e < CH * CH; e += THREADS) {
-        const int i = e >> 6, j = e & 63;
-        Tq[i * LD64 + j] = f2h((j >> 4) <= (i >> 4) ? Ts[i * LDF + j] * beta_s[j] : 0.0f);
     }
     __syncthreads();
 
-    // ---- W = T' (k e^G) and U = T' v
+    // ---- W = T' (k e^G) and U = T' v without the blocks of T below the diagonal: block forward substitution on
+    // R = [k e^G | v] (64 rows, 256 columns), held transposed in LDS ([column][row]: keT then VT) and solved in
+    // place, sixteen columns per tile, four tiles per wave, no barrier:
+    //   Z_a = -sum_{b<a} L_ab X_b,   X_a = T'_aa R_a + T_aa Z_a.
+    // R_a enters the last product unrounded (v is exact in fp16), so X is rounded once; Z, X_b and L are fp16.
     {
+        uint16_t* RT = keT;                       // [256][LD64]: VT follows keT
+        static_assert(I_VT == I_KET + DK * LD64 * 2, "R^T is keT and VT side by side");
+        uint16_t* Zs = reinterpret_cast<uint16_t*>(smem + I_Z);
         const int rl = 4 * (lane >> 4), cl = lane & 15;
         const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-        // W transposed: tile [16 keys][16 rows], so a lane ends with four consecutive keys of one row
 #pragma unroll
-        for (int mt = 2 * wave; mt < 2 * wave + 2; ++mt)
+        for (int a = 0; a < 4; ++a) {
+            const uint4 tt = frag(TT, LDT, SUB * a, 0, lane);
+            f32x4 z[4];
+            if (a > 0) {
+                const uint4 l0 = frag(Ln, LD64, SUB * a, 0, lane);
 #pragma unroll
-            for (int nt = 0; nt < 4; ++nt) {
-                const f32x4 acc = tile_f16(keT, SUB * mt, LD64, Tq, SUB * nt, LD64, CH, lane, zero);
-                const uint32_t w0 = (uint32_t)f2h(acc[0]) | ((uint32_t)f2h(acc[1]) << 16);
-                const uint32_t w1 = (uint32_t)f2h(acc[2]) | ((uint32_t)f2h(acc[3]) << 16);
-                *reinterpret_cast<uint2*>(wsc + WS_W + ((SUB * nt + cl) * DK + SUB * mt + rl) * 2) = make_uint2(w0, w1);
+                for (int q = 0; q < 4; ++q) z[q] = mfma_f16(frag(RT, LD64, SUB * (4 * wave + q), 0, lane), l0, zero);
+                if (a == 3) {
+                    const uint4 l1 = frag(Ln, LD64, SUB * a, 32, lane);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) z[q] = mfma_f16(frag(RT, LD64, SUB * (4 * wave + q), 32, lane), l1, z[q]);
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    uint16_t* zt = Zs + (4 * wave + q) * SUB * LDZ;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) zt[(rl + r) * LDZ + cl] = f2h(z[q][r]);
+                }
             }
-        // U: tile [16 rows][16 values], stored transposed: four consecutive rows of one value column
 #pragma unroll
-        for (int nt = 2 * wave; nt < 2 * wave + 2; ++nt)
+            for (int q = 0; q < 4; ++q) {
+                const int ct = 4 * wave + q;
+                // A operand [16 columns][K = 32]: k < 16 is R_a (lanes 0..31), k >= 16 is Z_a (lanes 32..63)
+                uint4 af;
+                if (lane < 32) {
+                    af = *reinterpret_cast<const uint4*>(RT + (SUB * ct + cl) * LD64 + SUB * a + 8 * (lane >> 4));
+                } else if (a > 0) {
+                    af = *reinterpret_cast<const uint4*>(Zs + ct * SUB * LDZ + cl * LDZ + 8 * ((lane >> 4) - 2));
+                } else {
+                    af = make_uint4(0u, 0u, 0u, 0u);
+                }
+                const f32x4 x = mfma_f16(af, tt, zero);
+                // X^T back in place of R^T_a: four columns rl.. of row 16 a + cl
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt) {
-                const f32x4 acc = tile_f16(Tq, SUB * mt, LD64, VT, SUB * nt, LD64, CH, lane, zero);
-                const uint32_t u0 = (uint32_t)f2h(acc[0]) | ((uint32_t)f2h(acc[1]) << 16);
-                const uint32_t u1 = (uint32_t)f2h(acc[2]) | ((uint32_t)f2h(acc[3]) << 16);
-                *reinterpret_cast<uint2*>(wsc + WS_UT + ((SUB * nt + cl) * CH + SUB * mt + rl) * 2) = make_uint2(u0, u1);
+                for (int r = 0; r < 4; ++r) RT[(SUB * ct + rl + r) * LD64 + SUB * a + cl] = f2h(x[r]);
+                if (ct < DK / SUB) {              // W [row][key]: four consecutive keys of one row
+                    const uint32_t w0 = (uint32_t)f2h(x[0]) | ((uint32_t)f2h(x[1]) << 16);
+                    const uint32_t w1 = (uint32_t)f2h(x[2]) | ((uint32_t)f2h(x[3]) << 16);
+                    *reinterpret_cast<uint2*>(wsc + WS_W + ((SUB * a + cl) * DK + SUB * ct + rl) * 2) = make_uint2(w0, w1);
+                }
             }
+        }
+    }
+    __syncthreads();
+    // U^T [value][row] is now what VT holds
+    for (int e = t; e < DV * (CH / 8); e += THREADS) {
+        const int v = e >> 3, piece = e & 7;
+        *reinterpret_cast<uint4*>(wsc + WS_UT + (v * CH + 8 * piece) * 2) =
+            *reinterpret_cast<const uint4*>(VT + v * LD64 + 8 * piece);
     }
 }
 
