@@ -103,7 +103,7 @@ constexpr int I_INV = I_BETA + CH * 4;            // f32 [2][64]: 1/|q| * 128^-0
 constexpr int I_KET = I_INV + 2 * CH * 4;         // fp16 [128 keys][LD64]: k e^G, transposed
 constexpr int I_VT = I_KET + DK * LD64 * 2;       // fp16 [128 values][LD64]: v, transposed
 constexpr int I_LN = I_VT + DV * LD64 * 2;        // fp16 [64][LD64]: -L below the block diagonal, zero elsewhere
-constexpr int LDD = SUB + 1;                      // f32 rows of a diagonal block of L
+constexpr int LDD = SUB + 4;                      // f32 row stride of a diagonal block of L (16-byte multiple)
 constexpr int I_LD = I_LN + CH * LD64 * 2;        // f32 [4][16][LDD]: the diagonal blocks of L
 constexpr int I_KC1 = I_LD + 4 * SUB * LDD * 4;   // fp16 [32][LD128]: column side around the chunk's middle
 constexpr int I_PASS = I_KC1 + 32 * LD128 * 2;    // the rest is reused by every half
@@ -126,6 +126,7 @@ constexpr int I_XIN = I_R2;                       // bf16 [3][35][LDX]
 constexpr int I_AIN = I_PASS;                     // bf16 [64][LDX]
 static_assert(I_XIN + 3 * XROWS * LDX * 2 <= I_END, "input staging must fit behind the diagonal operands");
 constexpr int INTRA_LDS = I_END;
+constexpr int INTRA_CPW = 4;                     // consecutive chunks of a head per intra workgroup
 static_assert(I_Z + 16 * SUB * LDZ * 2 <= I_END, "solve scratch must fit the per-half region");
 static_assert(INTRA_LDS <= 160 * 1024, "intra_kernel LDS");
 
@@ -177,16 +178,16 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         const bf16_t* __restrict__ cw, const float* __restrict__ a_log, const float* __restrict__ dt_bias, float lower,
         int vec, unsigned char* __restrict__ ws) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int c_first = blockIdx.x * INTRA_CPW, h = blockIdx.y, b = blockIdx.z;
     const RowRange rr = request_rows(cu_rows, b, rows1);
-    const int r0 = sub0 + c * CH;                 // the chunk's first row inside the request
-    const int n = min(CH, rr.rows - r0);          // its real rows
-    if (n <= 0) return;
-    const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
-    const int d = t & (DK - 1), s = t >> 7;       // this lane's channel, and which sub-chunk of a half it takes
+    if (rr.rows - (sub0 + c_first * CH) <= 0) return;
+    // t, and what derives from it, are re-made at the top of every chunk from a value the optimizer cannot see
+    // through: otherwise the hundreds of per-lane addresses of the body are hoisted out of the chunk loop and
+    // spill.
+    int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+    int d = t & (DK - 1), s = t >> 7;             // this lane's channel, and which sub-chunk of a half it takes
     const long long C = 3LL * H * DK;
     const bf16_t* cs = conv + (conv_off != nullptr ? conv_off[b] : 0);
-    unsigned char* wsc = ws + (((long long)b * H + h) * chunks + c) * (long long)WS_BYTES;
 
     float* tot = reinterpret_cast<float*>(smem + I_TOT);
     float* beta_s = reinterpret_cast<float*>(smem + I_BETA);
@@ -203,47 +204,35 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         if (rel >= rr.rows) return nullptr;
         return rel < 0 ? cs + (long long)(rel + WINDOW) * C : P + (rr.row0 + rel) * p_stride;
     };
-    // segment seg (q, k, v) of the input rows of half h2, three rows before its first included
-    auto x_src = [&](int h2, int seg) {
+    // segment seg (q, k, v) of the input rows of half h2 of the chunk starting at row first, three rows before
+    // the half's first included
+    auto x_src = [&](int first, int h2, int seg) {
         return [=](int j) -> const bf16_t* {
-            const bf16_t* row = input_row(r0 + 32 * h2 - WINDOW + j);
+            const bf16_t* row = input_row(first + 32 * h2 - WINDOW + j);
             return row != nullptr ? row + seg * H * DK + h * DK : nullptr;
         };
     };
-    auto a_src = [&](int R) -> const bf16_t* {
-        return R < n ? A + (rr.row0 + r0 + R) * a_stride + h * DK : nullptr;
+    auto a_src = [&](int first) {
+        return [=](int R) -> const bf16_t* {
+            return first + R < rr.rows ? A + (rr.row0 + first + R) * a_stride + h * DK : nullptr;
+        };
     };
-    // every global input of the first half goes out now; the second half's follows while the first computes
+    // A workgroup takes INTRA_CPW consecutive chunks of its head. Every global input of a chunk's first half is
+    // requested while the chunk before it is still being worked on (for the first chunk: now); the second half's
+    // follows while the first half computes.
     StagedRows<CH> a_st;
     StagedRows<XROWS> x_st[3];
-    a_st.load(a_src, vec != 0, t);
+    a_st.load(a_src(sub0 + c_first * CH), vec != 0, t);
 #pragma unroll
-    for (int seg = 0; seg < 3; ++seg) x_st[seg].load(x_src(0, seg), vec != 0, t);
-    uint16_t* ain = reinterpret_cast<uint16_t*>(smem + I_AIN);
-    a_st.store(ain, a_src, vec != 0, t);
-    __syncthreads();
+    for (int seg = 0; seg < 3; ++seg) x_st[seg].load(x_src(sub0 + c_first * CH, 0, seg), vec != 0, t);
+    // the beta logit of row t of the chunk (lanes 0..63), requested with the rest of the chunk's inputs
+    auto beta_logit = [&](int first) -> bf16_t {
+        const int R = first + (t & (CH - 1));
+        return R < rr.rows ? P[(rr.row0 + R) * p_stride + b_off + h] : (bf16_t)0;
+    };
+    bf16_t b_raw = beta_logit(sub0 + c_first * CH);
     const float rate = fast_exp(a_log[h]);
     const float dtb = dt_bias[h * DK + d];
-    float cg[2][SUB];                             // inclusive cumulative sums, sub-chunks s and 2 + s
-#pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2) {
-        const int a = 2 * h2 + s;
-        float run = 0.0f;
-#pragma unroll
-        for (int i = 0; i < SUB; ++i) {
-            const int R = SUB * a + i;
-            float g = 0.0f;
-            if (R < n) g = lower * fast_sigmoid(rate * (bf2f(ain[R * LDX + d]) + dtb));
-            run += g;
-            cg[h2][i] = run;
-        }
-        tot[a * DK + d] = run;
-    }
-    if (t < CH) {
-        float bv = 0.0f;
-        if (t < n) bv = bfround(fast_sigmoid(bf2f(P[(rr.row0 + r0 + t) * p_stride + b_off + h])));
-        beta_s[t] = bv;
-    }
     // conv weights of this lane's q, k and v channels
     const unsigned cq = (unsigned)(h * DK + d), ck = (unsigned)(H * DK + h * DK + d), cv = (unsigned)(2 * H * DK + h * DK + d);
     float wq[TAPS], wk[TAPS], wv[TAPS];
@@ -258,6 +247,38 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         wv[0] = __uint_as_float(c4.x << 16); wv[1] = __uint_as_float(c4.x & 0xffff0000u);
         wv[2] = __uint_as_float(c4.y << 16); wv[3] = __uint_as_float(c4.y & 0xffff0000u);
     }
+#pragma unroll 1
+    for (int c = c_first; c < min(chunks, c_first + INTRA_CPW); ++c) {
+    asm volatile("" : "+v"(t));
+    wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    lane = t & 63;
+    d = t & (DK - 1);
+    s = __builtin_amdgcn_readfirstlane(t >> 7);   // uniform inside a wave
+    const int r0 = sub0 + c * CH;                 // the chunk's first row inside the request
+    const int n = min(CH, rr.rows - r0);          // its real rows
+    if (n <= 0) break;
+    const bool more = c + 1 < min(chunks, c_first + INTRA_CPW) && rr.rows - (r0 + CH) > 0;
+    unsigned char* wsc = ws + (((long long)b * H + h) * chunks + c) * (long long)WS_BYTES;
+    uint16_t* ain = reinterpret_cast<uint16_t*>(smem + I_AIN);
+    a_st.store(ain, a_src(r0), vec != 0, t);
+    __syncthreads();
+    float cg[2][SUB];                             // inclusive cumulative sums, sub-chunks s and 2 + s
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+        const int a = 2 * h2 + s;
+        float run = 0.0f;
+#pragma unroll
+        for (int i = 0; i < SUB; ++i) {
+            // rows past the end have g = 0; evaluated for every row and masked (a branch here would serialize
+            // the sixteen LDS reads and transcendentals)
+            const int R = SUB * a + i;
+            const float gv = lower * fast_sigmoid(rate * (bf2f(ain[R * LDX + d]) + dtb));
+            run += __uint_as_float(__float_as_uint(gv) & (R < n ? 0xffffffffu : 0u));
+            cg[h2][i] = run;
+        }
+        tot[a * DK + d] = run;
+    }
+    if (t < CH) beta_s[t] = t < n ? bfround(fast_sigmoid(bf2f(b_raw))) : 0.0f;
     __syncthreads();
     // prefix and suffix totals of this lane's channel: B[a] = sum of tot over sub-chunks before a
     float Bp[5];
@@ -276,11 +297,16 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         // the half's input rows (three before its first row included) into LDS, q | k | v side by side
         uint16_t* xin = reinterpret_cast<uint16_t*>(smem + I_XIN);
 #pragma unroll
-        for (int seg = 0; seg < 3; ++seg) x_st[seg].store(xin + seg * XROWS * LDX, x_src(h2, seg), vec != 0, t);
+        for (int seg = 0; seg < 3; ++seg) x_st[seg].store(xin + seg * XROWS * LDX, x_src(r0, h2, seg), vec != 0, t);
         __syncthreads();
         if (h2 == 0) {
 #pragma unroll
-            for (int seg = 0; seg < 3; ++seg) x_st[seg].load(x_src(1, seg), vec != 0, t);
+            for (int seg = 0; seg < 3; ++seg) x_st[seg].load(x_src(r0, 1, seg), vec != 0, t);
+        } else if (more) {
+            b_raw = beta_logit(r0 + CH);
+            a_st.load(a_src(r0 + CH), vec != 0, t);
+#pragma unroll
+            for (int seg = 0; seg < 3; ++seg) x_st[seg].load(x_src(r0 + CH, 0, seg), vec != 0, t);
         }
         // conv + SiLU, one bf16 rounding, 16 rows of q, k, v
         float qr[SUB], kr[SUB];
@@ -288,32 +314,31 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
             const uint16_t* xq_l = xin + (SUB * s) * LDX + d;                 // row j of the lane's sub-chunk: + j * LDX
             const uint16_t* xk_l = xq_l + XROWS * LDX;
             const uint16_t* xv_l = xk_l + XROWS * LDX;
-            float xq[TAPS], xk[TAPS], xv[TAPS];
+            // all 19 input rows of the three channels into registers first: the stores below go to the same
+            // memory, and reads issued between them would each wait out a full LDS latency
+            float xq[SUB + WINDOW], xk[SUB + WINDOW], xv[SUB + WINDOW];
 #pragma unroll
-            for (int j = 0; j < WINDOW; ++j) {
-                xq[j + 1] = bf2f(xq_l[j * LDX]);
-                xk[j + 1] = bf2f(xk_l[j * LDX]);
-                xv[j + 1] = bf2f(xv_l[j * LDX]);
+            for (int j = 0; j < SUB + WINDOW; ++j) {
+                xq[j] = bf2f(xq_l[j * LDX]);
+                xk[j] = bf2f(xk_l[j * LDX]);
+                xv[j] = bf2f(xv_l[j * LDX]);
             }
             uint32_t vpack[SUB / 2];
 #pragma unroll
             for (int i = 0; i < SUB; ++i) {
-#pragma unroll
-                for (int j = 0; j < WINDOW; ++j) { xq[j] = xq[j + 1]; xk[j] = xk[j + 1]; xv[j] = xv[j + 1]; }
                 const bool live = SUB * a + i < n;
-                xq[3] = bf2f(xq_l[(WINDOW + i) * LDX]);
-                xk[3] = bf2f(xk_l[(WINDOW + i) * LDX]);
-                xv[3] = bf2f(xv_l[(WINDOW + i) * LDX]);
                 float aq = 0.0f, ak = 0.0f, av = 0.0f;
 #pragma unroll
                 for (int tap = 0; tap < TAPS; ++tap) {
-                    aq = __builtin_fmaf(wq[tap], xq[tap], aq);
-                    ak = __builtin_fmaf(wk[tap], xk[tap], ak);
-                    av = __builtin_fmaf(wv[tap], xv[tap], av);
+                    aq = __builtin_fmaf(wq[tap], xq[i + tap], aq);
+                    ak = __builtin_fmaf(wk[tap], xk[i + tap], ak);
+                    av = __builtin_fmaf(wv[tap], xv[i + tap], av);
                 }
-                const float sq = live ? bfround(aq * fast_sigmoid(aq)) : 0.0f;
-                const float sk = live ? bfround(ak * fast_sigmoid(ak)) : 0.0f;
-                const float sv = live ? bfround(av * fast_sigmoid(av)) : 0.0f;
+                // rows past the end give zero: masked, not branched around
+                const uint32_t keep = live ? 0xffffffffu : 0u;
+                const float sq = __uint_as_float(__float_as_uint(bfround(aq * fast_sigmoid(aq))) & keep);
+                const float sk = __uint_as_float(__float_as_uint(bfround(ak * fast_sigmoid(ak))) & keep);
+                const float sv = __uint_as_float(__float_as_uint(bfround(av * fast_sigmoid(av))) & keep);
                 qr[i] = sq;
                 kr[i] = sk;
                 rawq[(lr0 + i) * LD128 + d] = f2bf(sq);
@@ -373,10 +398,16 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
             // around the chunk's middle: columns of sub-chunk 0 still cross sub-chunk 1, rows of 3 crossed 2
             const float eMid = (a == 0) ? fast_exp(tot[1 * DK + d]) : (a == 3 ? fast_exp(tot[2 * DK + d]) : 1.0f);
             uint32_t kepack[SUB / 2], kgpack[SUB / 2];
+            float kinv[SUB], qinv[SUB];               // read before the stores below (same memory, see the conv)
+#pragma unroll
+            for (int i = 0; i < SUB; ++i) {
+                kinv[i] = inv_s[CH + SUB * a + i];
+                qinv[i] = inv_s[SUB * a + i];
+            }
 #pragma unroll
             for (int i = 0; i < SUB; ++i) {
                 const int R = SUB * a + i;
-                const float kh = kr[i] * inv_s[CH + R], qh = qr[i] * inv_s[R];
+                const float kh = kr[i] * kinv[i], qh = qr[i] * qinv[i];
                 const float e1 = fast_exp(cg[h2][i]);           // e^{G_i - G at the sub-chunk's start}
                 const float ep = e1 * eneg0;                    // e^{G_i - G_first}
                 const float rp = fast_rcp(ep);                  // e^{G_first - G_i}, up to e^87
@@ -514,47 +545,63 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         uint16_t* Zs = reinterpret_cast<uint16_t*>(smem + I_Z);
         const int rl = 4 * (lane >> 4), cl = lane & 15;
         const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        auto pack4 = [](const f32x4 v) {
+            return make_uint2((uint32_t)f2h(v[0]) | ((uint32_t)f2h(v[1]) << 16),
+                              (uint32_t)f2h(v[2]) | ((uint32_t)f2h(v[3]) << 16));
+        };
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const uint4 tt = frag(TT, LDT, SUB * a, 0, lane);
-            f32x4 z[4];
             if (a > 0) {
+                // Z tile [16 rows j][16 columns c]: a lane ends with four consecutive rows of one column
+                f32x4 z[4];
                 const uint4 l0 = frag(Ln, LD64, SUB * a, 0, lane);
 #pragma unroll
-                for (int q = 0; q < 4; ++q) z[q] = mfma_f16(frag(RT, LD64, SUB * (4 * wave + q), 0, lane), l0, zero);
+                for (int q = 0; q < 4; ++q) z[q] = mfma_f16(l0, frag(RT, LD64, SUB * (4 * wave + q), 0, lane), zero);
                 if (a == 3) {
                     const uint4 l1 = frag(Ln, LD64, SUB * a, 32, lane);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) z[q] = mfma_f16(frag(RT, LD64, SUB * (4 * wave + q), 32, lane), l1, z[q]);
+                    for (int q = 0; q < 4; ++q) z[q] = mfma_f16(l1, frag(RT, LD64, SUB * (4 * wave + q), 32, lane), z[q]);
                 }
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    uint16_t* zt = Zs + (4 * wave + q) * SUB * LDZ;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) zt[(rl + r) * LDZ + cl] = f2h(z[q][r]);
-                }
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<uint2*>(Zs + ((4 * wave + q) * SUB + cl) * LDZ + rl) = pack4(z[q]);
             }
+            // [R_a | Z_a] of a column tile as an operand [16 columns][K = 32]: k < 16 is R_a (lanes 0..31), k >= 16
+            // is Z_a (lanes 32..63): one read at a per-lane offset, no branch
+            uint4 rz[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int ct = 4 * wave + q;
-                // A operand [16 columns][K = 32]: k < 16 is R_a (lanes 0..31), k >= 16 is Z_a (lanes 32..63)
-                uint4 af;
-                if (lane < 32) {
-                    af = *reinterpret_cast<const uint4*>(RT + (SUB * ct + cl) * LD64 + SUB * a + 8 * (lane >> 4));
-                } else if (a > 0) {
-                    af = *reinterpret_cast<const uint4*>(Zs + ct * SUB * LDZ + cl * LDZ + 8 * ((lane >> 4) - 2));
-                } else {
-                    af = make_uint4(0u, 0u, 0u, 0u);
+                const int off_r = I_KET + ((SUB * ct + cl) * LD64 + SUB * a + 8 * (lane >> 4)) * 2;
+                const int off_z = I_Z + ((ct * SUB + cl) * LDZ + 8 * ((lane >> 4) - 2)) * 2;
+                rz[q] = *reinterpret_cast<const uint4*>(smem + (lane < 32 ? off_r : off_z));
+                if (a == 0) {                     // Z_0 = 0
+                    const uint32_t keep = lane < 32 ? 0xffffffffu : 0u;
+                    rz[q] = make_uint4(rz[q].x & keep, rz[q].y & keep, rz[q].z & keep, rz[q].w & keep);
                 }
-                const f32x4 x = mfma_f16(af, tt, zero);
-                // X^T back in place of R^T_a: four columns rl.. of row 16 a + cl
+            }
+            if (wave < 2) {
+                // key columns: X^T tile [16 keys][16 rows], so a lane ends with four consecutive keys of one row
+                // of W [row][key] for the workspace; back into R^T as four 16-bit pieces
+                f32x4 x[4];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) RT[(SUB * ct + rl + r) * LD64 + SUB * a + cl] = f2h(x[r]);
-                if (ct < DK / SUB) {              // W [row][key]: four consecutive keys of one row
-                    const uint32_t w0 = (uint32_t)f2h(x[0]) | ((uint32_t)f2h(x[1]) << 16);
-                    const uint32_t w1 = (uint32_t)f2h(x[2]) | ((uint32_t)f2h(x[3]) << 16);
-                    *reinterpret_cast<uint2*>(wsc + WS_W + ((SUB * a + cl) * DK + SUB * ct + rl) * 2) = make_uint2(w0, w1);
+                for (int q = 0; q < 4; ++q) x[q] = mfma_f16(rz[q], tt, zero);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int ct = 4 * wave + q;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) RT[(SUB * ct + rl + r) * LD64 + SUB * a + cl] = f2h(x[q][r]);
+                    *reinterpret_cast<uint2*>(wsc + WS_W + ((SUB * a + cl) * DK + SUB * ct + rl) * 2) = pack4(x[q]);
                 }
+            } else {
+                // value columns: X tile [16 rows][16 values]: four consecutive rows of one value, one piece of R^T
+                f32x4 x[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) x[q] = mfma_f16(tt, rz[q], zero);
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<uint2*>(RT + (SUB * (4 * wave + q) + cl) * LD64 + SUB * a + rl) = pack4(x[q]);
             }
         }
     }
@@ -564,6 +611,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         const int v = e >> 3, piece = e & 7;
         *reinterpret_cast<uint4*>(wsc + WS_UT + (v * CH + 8 * piece) * 2) =
             *reinterpret_cast<const uint4*>(VT + v * LD64 + 8 * piece);
+    }
+    __syncthreads();                              // the next chunk reuses every LDS region
     }
 }
 
@@ -892,7 +941,7 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
     const int step = (int)chunks * CH;
     for (int sub0 = 0; sub0 == 0 || sub0 < max_rows; sub0 += step) {
         if (max_rows > 0) {
-            intra_kernel<<<dim3((unsigned)chunks, heads, batch), THREADS, INTRA_LDS, st>>>(
+            intra_kernel<<<dim3((unsigned)((chunks + INTRA_CPW - 1) / INTRA_CPW), heads, batch), THREADS, INTRA_LDS, st>>>(
                 heads, cu_rows, rows1, sub0, (int)chunks, bfp(p), p_stride, b_off, bfp(a), a_stride, bfp(conv), coff,
                 bfp(conv_w), a_log, dt_bias, lower, vec, ws);
             const int rc = (int)hipGetLastError();
