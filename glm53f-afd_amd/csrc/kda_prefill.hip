@@ -1,5 +1,5 @@
 // KDA chunked prefill on gfx950: the delta rule over a prompt segment in the chunked (WY/UT) form, with every
-// GEMM-shaped step on the matrix cores (v_mfma_f32_16x16x32_{f16,bf16}, f32 accumulation).
+// GEMM-shaped step on the matrix cores (v_mfma_f32_16x16x32_f16 and, for a few tiles, v_mfma_f32_16x16x4_f32).
 //
 // The algebra is the reference's chunk form (crates/glm53f-kda/src/chunked.rs:67-198; kernel counterpart
 // kda_prefill.cu:95-538 with 16-row chunks on CUDA cores). Here a chunk is 64 rows in four sub-chunks of 16.
@@ -9,10 +9,10 @@
 //   from the state S entering the chunk: V' = U - W S,  Y = Qg S + M V',  S <- e^{G_last} S + Kg^T V'.
 // e^{G_i - G_j} is factored around a reference row so that both factors are GEMM operands:
 //   * inside a sub-chunk (diagonal 16x16 blocks) around the sub-chunk's first row; one factor reaches e^{+87}
-//     (15 rows at the -5.8 bound), so these operands are bf16 split into hi + lo (three products);
+//     (15 rows at the -5.8 bound), beyond fp16, so these few tiles run on the f32 MFMA with f32 operands;
 //   * between sub-chunks around a row in between (the end of a sub-chunk, or the middle of the chunk), where
 //     both exponents are <= 0 and the operands are fp16 (11-bit mantissa at the bf16 MFMA rate).
-// Everything that feeds the state is fp16 or split bf16. Only the diagonal 16x16 blocks of T are formed (in f32);
+// Everything that feeds the state is fp16 or f32. Only the diagonal 16x16 blocks of T are formed (in f32);
 // W and U come from a block forward substitution on [k e^G | v] with MFMA tiles (see intra_kernel).
 //
 // Kernels per pass: intra_kernel (one workgroup per chunk, head, request: prologue + L, M, T, W, U, Qg, Kg into
@@ -31,7 +31,6 @@ constexpr int VBLOCKS = DV / NV;          // inter workgroups per head
 
 typedef _Float16 f16_t;
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // a register-friendly 128-bit piece
 
@@ -65,10 +64,6 @@ __device__ __forceinline__ uint4 frag(const uint16_t* base, int ld, int row0, in
 __device__ __forceinline__ f32x4 mfma_f16(uint4 a, uint4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
-__device__ __forceinline__ f32x4 mfma_bf16(uint4 a, uint4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0,
-                                                   0);
-}
 
 // C[16][16] += A[a_row0 ..][0, K) . B^T[b_row0 ..][0, K) with fp16 operands.
 __device__ __forceinline__ f32x4 tile_f16(const uint16_t* a, int a_row0, int lda, const uint16_t* b, int b_row0, int ldb,
@@ -77,23 +72,20 @@ __device__ __forceinline__ f32x4 tile_f16(const uint16_t* a, int a_row0, int lda
     return acc;
 }
 
-// The same with bf16 operands split into hi + lo: a_hi b_hi + a_hi b_lo + a_lo b_hi.
-__device__ __forceinline__ f32x4 tile_bf16x3(const uint16_t* ah, const uint16_t* al, int a_row0, const uint16_t* bh,
-                                             const uint16_t* bl, int b_row0, int lane, f32x4 acc) {
-    for (int k0 = 0; k0 < DK; k0 += 32) {
-        const uint4 fah = frag(ah, LD128, a_row0, k0, lane), fal = frag(al, LD128, a_row0, k0, lane);
-        const uint4 fbh = frag(bh, LD128, b_row0, k0, lane), fbl = frag(bl, LD128, b_row0, k0, lane);
-        acc = mfma_bf16(fal, fbh, acc);
-        acc = mfma_bf16(fah, fbl, acc);
-        acc = mfma_bf16(fah, fbh, acc);
+// C[16][16] += A[a_row0 ..][0, 128) . B^T[b_row0 ..][0, 128) with f32 operands (v_mfma_f32_16x16x4_f32: lanes
+// 16 g .. 16 g + 15 supply one k per instruction). Which k a lane group supplies at which step is free as long as
+// both operands agree, so group g walks k = 32 g .. 32 g + 31 and reads its 32 values as eight 128-bit pieces.
+constexpr int LDG = DK + 4;                       // f32 row stride of these operands
+__device__ __forceinline__ f32x4 tile_f32(const float* a, int a_row0, const float* b, int b_row0, int lane, f32x4 acc) {
+    const f32x4* pa = reinterpret_cast<const f32x4*>(a + (a_row0 + (lane & 15)) * LDG + 32 * (lane >> 4));
+    const f32x4* pb = reinterpret_cast<const f32x4*>(b + (b_row0 + (lane & 15)) * LDG + 32 * (lane >> 4));
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+        const f32x4 va = pa[p], vb = pb[p];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(va[e], vb[e], acc, 0, 0, 0);
     }
     return acc;
-}
-
-// bf16 hi + lo of x: hi = bf16(x), lo = bf16(x - hi).
-__device__ __forceinline__ void split_bf16(float x, uint16_t& hi, uint16_t& lo) {
-    hi = f2bf(x);
-    lo = f2bf(x - bf2f(hi));
 }
 
 // LDS map of intra_kernel, bytes.
@@ -109,7 +101,7 @@ constexpr int I_KC1 = I_LD + 4 * SUB * LDD * 4;   // fp16 [32][LD128]: column si
 constexpr int I_PASS = I_KC1 + 32 * LD128 * 2;    // the rest is reused by every half
 constexpr int P_ROWS32 = 32 * LD128 * 2;          // one [32][LD128] 16-bit array
 constexpr int P_ROWS16 = 16 * LD128 * 2;
-constexpr int I_DIAG = I_PASS;                    // six [32][LD128] bf16 arrays: KrD hi/lo, QrD hi/lo, KcD hi/lo
+constexpr int I_DIAG = I_PASS;                    // three f32 [32][LDG] arrays: KrD, QrD, KcD (within six P_ROWS32)
 constexpr int I_RAWQ = I_PASS;                    // raw q, k (bf16) before the norms: dead before the operands land
 constexpr int I_RAWK = I_PASS + P_ROWS32;
 constexpr int I_R2 = I_DIAG + 6 * P_ROWS32;       // KR2, QR2, KC2: three [16][LD128] fp16 arrays
@@ -125,6 +117,7 @@ constexpr int XROWS = 32 + WINDOW;
 constexpr int I_XIN = I_R2;                       // bf16 [3][35][LDX]
 constexpr int I_AIN = I_PASS;                     // bf16 [64][LDX]
 static_assert(I_XIN + 3 * XROWS * LDX * 2 <= I_END, "input staging must fit behind the diagonal operands");
+static_assert(3 * 32 * LDG * 4 <= 6 * P_ROWS32, "the f32 diagonal operands fit their region");
 constexpr int INTRA_LDS = I_END;
 constexpr int INTRA_CPW = 4;                     // consecutive chunks of a head per intra workgroup
 static_assert(I_Z + 16 * SUB * LDZ * 2 <= I_END, "solve scratch must fit the per-half region");
@@ -326,7 +319,6 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
             uint32_t vpack[SUB / 2];
 #pragma unroll
             for (int i = 0; i < SUB; ++i) {
-                const bool live = SUB * a + i < n;
                 float aq = 0.0f, ak = 0.0f, av = 0.0f;
 #pragma unroll
                 for (int tap = 0; tap < TAPS; ++tap) {
@@ -334,15 +326,14 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
                     ak = __builtin_fmaf(wk[tap], xk[i + tap], ak);
                     av = __builtin_fmaf(wv[tap], xv[i + tap], av);
                 }
-                // rows past the end give zero: masked, not branched around
-                const uint32_t keep = live ? 0xffffffffu : 0u;
-                const float sq = __uint_as_float(__float_as_uint(bfround(aq * fast_sigmoid(aq))) & keep);
-                const float sk = __uint_as_float(__float_as_uint(bfround(ak * fast_sigmoid(ak))) & keep);
-                const float sv = __uint_as_float(__float_as_uint(bfround(av * fast_sigmoid(av))) & keep);
-                qr[i] = sq;
-                kr[i] = sk;
-                rawq[(lr0 + i) * LD128 + d] = f2bf(sq);
-                rawk[(lr0 + i) * LD128 + d] = f2bf(sk);
+                // Rows past the request's end are not masked: their beta is zero, which removes them from L, W, U
+                // and the state update, and their outputs are never stored.
+                const uint16_t qb = f2bf(aq * fast_sigmoid(aq)), kb = f2bf(ak * fast_sigmoid(ak));
+                const float sv = bfround(av * fast_sigmoid(av));
+                qr[i] = bf2f(qb);
+                kr[i] = bf2f(kb);
+                rawq[(lr0 + i) * LD128 + d] = qb;
+                rawk[(lr0 + i) * LD128 + d] = kb;
                 const uint32_t hv = f2h(sv);        // a bf16 value is exact in fp16 (but for values below 2^-14)
                 if (i & 1) vpack[i / 2] |= hv << 16; else vpack[i / 2] = hv;
             }
@@ -379,12 +370,9 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         __syncthreads();
         // operands of this lane's 16 rows
         {
-            uint16_t* KrDh = reinterpret_cast<uint16_t*>(smem + I_DIAG);
-            uint16_t* KrDl = KrDh + 32 * LD128;
-            uint16_t* QrDh = KrDl + 32 * LD128;
-            uint16_t* QrDl = QrDh + 32 * LD128;
-            uint16_t* KcDh = QrDl + 32 * LD128;
-            uint16_t* KcDl = KcDh + 32 * LD128;
+            float* KrD = reinterpret_cast<float*>(smem + I_DIAG);
+            float* QrD = KrD + 32 * LDG;
+            float* KcD = QrD + 32 * LDG;
             uint16_t* KR2 = reinterpret_cast<uint16_t*>(smem + I_R2);
             uint16_t* QR2 = KR2 + 16 * LD128;
             uint16_t* KC2 = QR2 + 16 * LD128;
@@ -413,10 +401,9 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
                 const float rp = fast_rcp(ep);                  // e^{G_first - G_i}, up to e^87
                 const float col2 = ep_last * rp;                // e^{G at the sub-chunk's end - G_i}
                 const int lr = lr0 + i;
-                uint16_t hi, lo;
-                split_bf16(kh * ep, hi, lo); KrDh[lr * LD128 + d] = hi; KrDl[lr * LD128 + d] = lo;
-                split_bf16(qh * ep, hi, lo); QrDh[lr * LD128 + d] = hi; QrDl[lr * LD128 + d] = lo;
-                split_bf16(kh * rp, hi, lo); KcDh[lr * LD128 + d] = hi; KcDl[lr * LD128 + d] = lo;
+                KrD[lr * LDG + d] = kh * ep;
+                QrD[lr * LDG + d] = qh * ep;
+                KcD[lr * LDG + d] = kh * rp;
                 if (s == 1) {
                     KR2[i * LD128 + d] = f2h(kh * e1);
                     QR2[i * LD128 + d] = f2h(qh * e1);
@@ -444,12 +431,9 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         __syncthreads();
         // the half's blocks of L and M on the matrix cores
         {
-            const uint16_t* KrDh = reinterpret_cast<const uint16_t*>(smem + I_DIAG);
-            const uint16_t* KrDl = KrDh + 32 * LD128;
-            const uint16_t* QrDh = KrDl + 32 * LD128;
-            const uint16_t* QrDl = QrDh + 32 * LD128;
-            const uint16_t* KcDh = QrDl + 32 * LD128;
-            const uint16_t* KcDl = KcDh + 32 * LD128;
+            const float* KrD = reinterpret_cast<const float*>(smem + I_DIAG);
+            const float* QrD = KrD + 32 * LDG;
+            const float* KcD = QrD + 32 * LDG;
             const uint16_t* KR2 = reinterpret_cast<const uint16_t*>(smem + I_R2);
             const uint16_t* QR2 = KR2 + 16 * LD128;
             const uint16_t* KC2 = QR2 + 16 * LD128;
@@ -484,8 +468,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
             // diagonal blocks: waves 0, 1 take L of sub-chunks 2 h2, 2 h2 + 1; waves 2, 3 take M
             {
                 const int sub = wave & 1, blk = 2 * h2 + sub;
-                if (wave < 2) put_L(tile_bf16x3(KrDh, KrDl, SUB * sub, KcDh, KcDl, SUB * sub, lane, zero), blk, blk);
-                else put_M(tile_bf16x3(QrDh, QrDl, SUB * sub, KcDh, KcDl, SUB * sub, lane, zero), blk, blk);
+                if (wave < 2) put_L(tile_f32(KrD, SUB * sub, KcD, SUB * sub, lane, zero), blk, blk);
+                else put_M(tile_f32(QrD, SUB * sub, KcD, SUB * sub, lane, zero), blk, blk);
             }
             // the block between the half's two sub-chunks
             if (wave == 0) put_L(tile_f16(KR2, 0, LD128, KC2, 0, LD128, DK, lane, zero), 2 * h2 + 1, 2 * h2);
@@ -623,7 +607,8 @@ constexpr int N_K = N_Q + CH * LD128 * 2;         // fp16 [128][LD64]: Kg transp
 constexpr int N_M = N_K + DK * LD64 * 2;          // fp16 [64][LD64]
 constexpr int N_U = N_M + CH * LD64 * 2;          // fp16 [NV][LD64]: this block's columns of U, transposed
 constexpr int N_E = N_U + NV * LD64 * 2;          // f32 [128]
-constexpr int N_S = N_E + DK * 4;                 // fp16 [NV][LD128]: the state, transposed
+constexpr int N_BUF = N_E + DK * 4;               // one chunk's staged workspace; two of them, used alternately
+constexpr int N_S = 2 * N_BUF;                    // fp16 [NV][LD128]: the state, transposed
 constexpr int N_V = N_S + NV * LD128 * 2;         // fp16 [NV][LD64]: V', transposed
 constexpr int INTER_LDS = N_V + NV * LD64 * 2;
 static_assert(INTER_LDS <= 160 * 1024, "inter_kernel LDS");
@@ -673,12 +658,6 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
     const long long sbase = (state_off != nullptr ? state_off[b] : 0) + (long long)h * DV * DK;
     const int rl = 4 * (lane >> 4), cl = lane & 15;
 
-    uint16_t* Wl = reinterpret_cast<uint16_t*>(smem + N_W);
-    uint16_t* Ql = reinterpret_cast<uint16_t*>(smem + N_Q);
-    uint16_t* Kl = reinterpret_cast<uint16_t*>(smem + N_K);
-    uint16_t* Ml = reinterpret_cast<uint16_t*>(smem + N_M);
-    uint16_t* Ul = reinterpret_cast<uint16_t*>(smem + N_U);
-    float* El = reinterpret_cast<float*>(smem + N_E);
     uint16_t* Sl = reinterpret_cast<uint16_t*>(smem + N_S);
     uint16_t* Vl = reinterpret_cast<uint16_t*>(smem + N_V);
 
@@ -694,38 +673,52 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         }
 
     const unsigned char* wsh = ws + ((long long)b * H + h) * chunks * (long long)WS_BYTES;
-    // Staging of a chunk's workspace: global -> registers (issued a chunk ahead) -> LDS. Every piece index q
-    // has its own array, so source and destination are compile-time functions of q: W (q 0-3), Qg (4-7),
-    // Kg^T (8-11), M (12-13), this block's rows of U^T (14), e^{G_last} (15, 32 lanes).
+    // Staging of a chunk's workspace: global -> registers -> LDS, two chunks deep at both levels. While chunk c is
+    // computed from LDS buffer c % 2, chunk c + 1 moves from its registers into the other buffer and chunk c + 2
+    // is requested into the registers chunk c came from. Every piece index q has its own array element, so source
+    // and destination are compile-time functions of q: W (q 0-3), Qg (4-7), Kg^T (8-11), M (12-13), this block's
+    // rows of U^T (14), e^{G_last} (15, 32 lanes).
     static_assert(STAGE_PER_LANE == 16 && NV == 32, "staging map");
-    u32x4 stage[STAGE_PER_LANE];
+    u32x4 stage_a[STAGE_PER_LANE], stage_b[STAGE_PER_LANE];
     const unsigned stage_lo = (unsigned)t * 16u;
-#define KDA_STAGE_LOAD(C_)                                                                                          \
+    // The sixteen loads of a chunk go out in four groups spread over a chunk's phases (PART_ 0..3: W, Qg, Kg^T, the
+    // rest): sixty-four kilobytes per workgroup take the vector memory pipeline longer to accept than a phase
+    // lasts, and a wave that issues them back to back stalls on the full queue.
+#define KDA_STAGE_LOAD(ST_, C_, PART_)                                                                              \
     {                                                                                                               \
         const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                               \
-        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                                             \
-            stage[q] = *reinterpret_cast<const u32x4*>(src_ + WS_W + q * 4096 + stage_lo);                           \
-            stage[4 + q] = *reinterpret_cast<const u32x4*>(src_ + WS_QG + q * 4096 + stage_lo);                      \
-            stage[8 + q] = *reinterpret_cast<const u32x4*>(src_ + WS_KGT + q * 4096 + stage_lo);                     \
+        if ((PART_) == 0) {                                                                                         \
+            _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                           \
+                ST_[q] = *reinterpret_cast<const u32x4*>(src_ + WS_W + q * 4096 + stage_lo);                         \
+        } else if ((PART_) == 1) {                                                                                  \
+            _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                           \
+                ST_[4 + q] = *reinterpret_cast<const u32x4*>(src_ + WS_QG + q * 4096 + stage_lo);                    \
+        } else if ((PART_) == 2) {                                                                                  \
+            _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                           \
+                ST_[8 + q] = *reinterpret_cast<const u32x4*>(src_ + WS_KGT + q * 4096 + stage_lo);                   \
+        } else {                                                                                                    \
+            ST_[12] = *reinterpret_cast<const u32x4*>(src_ + WS_M + stage_lo);                                      \
+            ST_[13] = *reinterpret_cast<const u32x4*>(src_ + WS_M + 4096 + stage_lo);                               \
+            ST_[14] = *reinterpret_cast<const u32x4*>(src_ + WS_UT + NV * vb * CH * 2 + stage_lo);                  \
+            ST_[15] = *reinterpret_cast<const u32x4*>(src_ + WS_E + (stage_lo & 511u));                             \
         }                                                                                                           \
-        stage[12] = *reinterpret_cast<const u32x4*>(src_ + WS_M + stage_lo);                                        \
-        stage[13] = *reinterpret_cast<const u32x4*>(src_ + WS_M + 4096 + stage_lo);                                 \
-        stage[14] = *reinterpret_cast<const u32x4*>(src_ + WS_UT + NV * vb * CH * 2 + stage_lo);                    \
-        stage[15] = *reinterpret_cast<const u32x4*>(src_ + WS_E + (stage_lo & 511u));                               \
     }
+#define KDA_STAGE_LOAD_ALL(ST_, C_)                                                                                 \
+    KDA_STAGE_LOAD(ST_, C_, 0) KDA_STAGE_LOAD(ST_, C_, 1) KDA_STAGE_LOAD(ST_, C_, 2) KDA_STAGE_LOAD(ST_, C_, 3)
     // 128-wide rows take 16 pieces each, 64-wide rows 8
-#define KDA_STAGE_STORE()                                                                                           \
+#define KDA_STAGE_STORE(ST_, BUF_)                                                                                  \
     {                                                                                                               \
+        unsigned char* buf_ = smem + (BUF_) * N_BUF;                                                                \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                                             \
             const int v_ = q * THREADS + t;                                                                         \
-            *reinterpret_cast<u32x4*>(Wl + (v_ >> 4) * LD128 + (v_ & 15) * 8) = stage[q];                            \
-            *reinterpret_cast<u32x4*>(Ql + (v_ >> 4) * LD128 + (v_ & 15) * 8) = stage[4 + q];                        \
-            *reinterpret_cast<u32x4*>(Kl + (v_ >> 3) * LD64 + (v_ & 7) * 8) = stage[8 + q];                          \
+            *reinterpret_cast<u32x4*>(buf_ + N_W + ((v_ >> 4) * LD128 + (v_ & 15) * 8) * 2) = ST_[q];                \
+            *reinterpret_cast<u32x4*>(buf_ + N_Q + ((v_ >> 4) * LD128 + (v_ & 15) * 8) * 2) = ST_[4 + q];            \
+            *reinterpret_cast<u32x4*>(buf_ + N_K + ((v_ >> 3) * LD64 + (v_ & 7) * 8) * 2) = ST_[8 + q];              \
         }                                                                                                           \
-        *reinterpret_cast<u32x4*>(Ml + (t >> 3) * LD64 + (t & 7) * 8) = stage[12];                                  \
-        *reinterpret_cast<u32x4*>(Ml + ((THREADS + t) >> 3) * LD64 + (t & 7) * 8) = stage[13];                      \
-        *reinterpret_cast<u32x4*>(Ul + (t >> 3) * LD64 + (t & 7) * 8) = stage[14];                                  \
-        if (t < 32) *reinterpret_cast<u32x4*>(El + t * 4) = stage[15];                                              \
+        *reinterpret_cast<u32x4*>(buf_ + N_M + ((t >> 3) * LD64 + (t & 7) * 8) * 2) = ST_[12];                      \
+        *reinterpret_cast<u32x4*>(buf_ + N_M + (((THREADS + t) >> 3) * LD64 + (t & 7) * 8) * 2) = ST_[13];          \
+        *reinterpret_cast<u32x4*>(buf_ + N_U + ((t >> 3) * LD64 + (t & 7) * 8) * 2) = ST_[14];                      \
+        if (t < 32) *reinterpret_cast<u32x4*>(buf_ + N_E + t * 16) = ST_[15];                                       \
     }
     // S^T for the first chunk
     auto put_state = [&]() {
@@ -739,13 +732,24 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
             }
     };
 
-    if (nch > 0) KDA_STAGE_LOAD(0)
-    for (int c = 0; c < nch; ++c) {
+    // Chunk c from LDS buffer `buf`. `mine` are the registers its workspace came through: free now, they take
+    // chunk c + 2; `next` hold chunk c + 1, which goes to the other buffer. Both moves are unconditional (past the
+    // end they repeat the last chunk, unused), so that the wait for `next` can be counted in loads still in flight.
+    auto chunk_step = [&](const int c, const int buf, u32x4 (&mine)[STAGE_PER_LANE], u32x4 (&next)[STAGE_PER_LANE])
+                          __attribute__((always_inline)) {
         const int nrows = min(CH, left - c * CH);
-        KDA_STAGE_STORE()
+        const uint16_t* Wl = reinterpret_cast<const uint16_t*>(smem + buf * N_BUF + N_W);
+        const uint16_t* Ql = reinterpret_cast<const uint16_t*>(smem + buf * N_BUF + N_Q);
+        const uint16_t* Kl = reinterpret_cast<const uint16_t*>(smem + buf * N_BUF + N_K);
+        const uint16_t* Ml = reinterpret_cast<const uint16_t*>(smem + buf * N_BUF + N_M);
+        const uint16_t* Ul = reinterpret_cast<const uint16_t*>(smem + buf * N_BUF + N_U);
+        const float* El = reinterpret_cast<const float*>(smem + buf * N_BUF + N_E);
         put_state();
-        __syncthreads();
-        if (c + 1 < nch) KDA_STAGE_LOAD(c + 1)
+        __syncthreads();      // the state and (stored during the chunk before) this chunk's workspace are in LDS;
+                              // every wave is done with the chunk before, so the other buffer, S and V' are free
+        const int c2 = min(c + 2, nch - 1);
+        KDA_STAGE_STORE(next, 1 - buf)
+        KDA_STAGE_LOAD(mine, c2, 0)
         const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
         // V' = U - W S: wave w takes rows 16 w .. 16 w + 15
         uint4 sfrag[2][4];
@@ -753,6 +757,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) sfrag[nt][ks] = frag(Sl, LD128, SUB * nt, 32 * ks, lane);
+        KDA_STAGE_LOAD(mine, c2, 1)
         f32x4 accV[2] = {zero, zero};
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
@@ -776,6 +781,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) vfrag[nt][ks] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
+        KDA_STAGE_LOAD(mine, c2, 2)
         f32x4 accY[2] = {zero, zero};
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
@@ -789,6 +795,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt) accY[nt] = mfma_f16(a, vfrag[nt][ks], accY[nt]);
         }
+        KDA_STAGE_LOAD(mine, c2, 3)
         {
             const long long grow0 = rr.row0 + sub0 + c * CH;
 #pragma unroll
@@ -825,7 +832,19 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
 #pragma unroll
                     for (int r = 0; r < 4; ++r) accS[mt][nt][r] = bfround(accS[mt][nt][r]);
         }
-        __syncthreads();
+    };
+    if (nch > 0) {
+        KDA_STAGE_LOAD_ALL(stage_a, 0)
+        KDA_STAGE_LOAD_ALL(stage_b, min(1, nch - 1))
+        KDA_STAGE_STORE(stage_a, 0)
+        // in pairs, so that the register sets and LDS buffers are compile-time choices; an odd last chunk follows
+        int c = 0;
+#pragma unroll 1
+        for (; c + 1 < nch; c += 2) {
+            chunk_step(c, 0, stage_a, stage_b);
+            chunk_step(c + 1, 1, stage_b, stage_a);
+        }
+        if (c < nch) chunk_step(c, 0, stage_a, stage_b);
     }
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
