@@ -35,13 +35,17 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // a register-friendly 128-bit piece
 
 // Workspace of one (request, head, chunk), bytes.
-constexpr int WS_W = 0;                   // fp16 [64 rows][128 keys]
+// Matrices that are MFMA operands of inter_kernel are stored in panels of 32 along their contraction index
+// ([panel][row][32]), so that the 16 rows x 32 of one operand fragment are 1 KiB of consecutive bytes.
+constexpr int WS_W = 0;                   // fp16 [4 key panels][64 rows][32 keys]
 constexpr int WS_UT = 16384;              // fp16 [128 values][64 rows]
-constexpr int WS_QG = 32768;              // fp16 [64 rows][128 keys]
-constexpr int WS_KGT = 49152;             // fp16 [128 keys][64 rows]
-constexpr int WS_M = 65536;               // fp16 [64 rows][64 rows]
+constexpr int WS_QG = 32768;              // fp16 [4 key panels][64 rows][32 keys]
+constexpr int WS_KGT = 49152;             // fp16 [2 row panels][128 keys][32 rows]
+constexpr int WS_M = 65536;               // fp16 [2 column panels][64 rows][32 columns]
 constexpr int WS_E = 73728;               // f32 [128 keys]: e^{G_last}
 constexpr int WS_BYTES = 74240;
+// Element index of (row, k) in a panelled matrix with `rows` rows.
+__device__ __forceinline__ int panel_index(int rows, int row, int k) { return ((k >> 5) * rows + row) * 32 + (k & 31); }
 
 // LDS row strides in 16-bit elements: 128- and 64-wide operand rows padded by 16 bytes, so that the sixteen
 // rows one MFMA fragment read touches fall into distinct banks.
@@ -419,12 +423,12 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
                 const uint32_t ke = f2h(kh * e1 * eB), kg = f2h(kh * col2 * eSuf);
                 if (i & 1) { kepack[i / 2] |= ke << 16; kgpack[i / 2] |= kg << 16; }
                 else { kepack[i / 2] = ke; kgpack[i / 2] = kg; }
-                reinterpret_cast<uint16_t*>(wsc + WS_QG)[R * DK + d] = f2h(qh * e1 * eB);
+                reinterpret_cast<uint16_t*>(wsc + WS_QG)[panel_index(CH, R, d)] = f2h(qh * e1 * eB);
             }
             uint4* kd = reinterpret_cast<uint4*>(keT + d * LD64 + SUB * a);
             kd[0] = make_uint4(kepack[0], kepack[1], kepack[2], kepack[3]);
             kd[1] = make_uint4(kepack[4], kepack[5], kepack[6], kepack[7]);
-            uint4* gd = reinterpret_cast<uint4*>(wsc + WS_KGT + (d * CH + SUB * a) * 2);
+            uint4* gd = reinterpret_cast<uint4*>(wsc + WS_KGT + panel_index(DK, d, SUB * a) * 2);
             gd[0] = make_uint4(kgpack[0], kgpack[1], kgpack[2], kgpack[3]);
             gd[1] = make_uint4(kgpack[4], kgpack[5], kgpack[6], kgpack[7]);
         }
@@ -461,7 +465,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int gi = SUB * rb + rl + r, gj = SUB * cb + cl;
-                    Mg[gi * CH + gj] = f2h((rb != cb || gj <= gi) ? acc[r] : 0.0f);
+                    Mg[panel_index(CH, gi, gj)] = f2h((rb != cb || gj <= gi) ? acc[r] : 0.0f);
                 }
             };
             const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -494,7 +498,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
             const int blk = e >> 8, r = (e >> 4) & 15, cc = e & 15;
             const int rb = blk < 3 ? 0 : (blk < 5 ? 1 : 2);
             const int cb = blk < 3 ? blk + 1 : (blk < 5 ? blk - 1 : 3);
-            Mg[(SUB * rb + r) * CH + SUB * cb + cc] = 0;
+            Mg[panel_index(CH, SUB * rb + r, SUB * cb + cc)] = 0;
             Ln[(SUB * rb + r) * LD64 + SUB * cb + cc] = 0;
         }
     }
@@ -576,7 +580,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
                     const int ct = 4 * wave + q;
 #pragma unroll
                     for (int r = 0; r < 4; ++r) RT[(SUB * ct + rl + r) * LD64 + SUB * a + cl] = f2h(x[q][r]);
-                    *reinterpret_cast<uint2*>(wsc + WS_W + ((SUB * a + cl) * DK + SUB * ct + rl) * 2) = pack4(x[q]);
+                    *reinterpret_cast<uint2*>(wsc + WS_W + panel_index(CH, SUB * a + cl, SUB * ct + rl) * 2) = pack4(x[q]);
                 }
             } else {
                 // value columns: X tile [16 rows][16 values]: four consecutive rows of one value, one piece of R^T
@@ -600,21 +604,10 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
     }
 }
 
-// LDS map of inter_kernel, bytes.
-constexpr int N_W = 0;                            // fp16 [64][LD128]
-constexpr int N_Q = N_W + CH * LD128 * 2;         // fp16 [64][LD128]
-constexpr int N_K = N_Q + CH * LD128 * 2;         // fp16 [128][LD64]: Kg transposed
-constexpr int N_M = N_K + DK * LD64 * 2;          // fp16 [64][LD64]
-constexpr int N_U = N_M + CH * LD64 * 2;          // fp16 [NV][LD64]: this block's columns of U, transposed
-constexpr int N_E = N_U + NV * LD64 * 2;          // f32 [128]
-constexpr int N_BUF = N_E + DK * 4;               // one chunk's staged workspace; two of them, used alternately
-constexpr int N_S = 2 * N_BUF;                    // fp16 [NV][LD128]: the state, transposed
+// LDS map of inter_kernel, bytes: only what the waves share.
+constexpr int N_S = 0;                            // fp16 [NV][LD128]: the state, transposed
 constexpr int N_V = N_S + NV * LD128 * 2;         // fp16 [NV][LD64]: V', transposed
 constexpr int INTER_LDS = N_V + NV * LD64 * 2;
-static_assert(INTER_LDS <= 160 * 1024, "inter_kernel LDS");
-// 16-byte pieces of one chunk's workspace a workgroup stages: W, Qg, Kg^T, M, its slice of U^T, e^{G_last}.
-constexpr int STAGE_VEC = (16384 + 16384 + 16384 + 8192 + NV * CH * 2 + 512) / 16;
-constexpr int STAGE_PER_LANE = (STAGE_VEC + THREADS - 1) / THREADS;
 
 template <typename S>
 __device__ __forceinline__ float load_state_elem4(const S* p, float (&v)[4]);
@@ -638,10 +631,21 @@ __device__ __forceinline__ void store_state_elem4(bf16_t* p, const f32x4 v) {
     *reinterpret_cast<uint2*>(p) = make_uint2(f2bf2(v[0], v[1]), f2bf2(v[2], v[3]));
 }
 
+// One chunk's operands of inter_kernel as a wave holds them: MFMA fragments straight from the workspace. Wave w
+// owns rows 16 w .. 16 w + 15 of the chunk (W, Qg, M, U) and keys 32 w .. 32 w + 31 of the state (Kg, e^{G_last}),
+// and nothing it loads is used by another wave, so none of it passes through LDS.
+struct InterOperands {
+    u32x4 w[4], q[4];                             // rows 16 w + l % 16, keys 32 ks + 8 (l / 16) ..
+    u32x4 m[2];                                   // rows 16 w + l % 16, chunk rows 32 ks + 8 (l / 16) ..
+    u32x4 k[2][2];                                // keys 32 w + 16 mt + l % 16, chunk rows 32 ks + 8 (l / 16) ..
+    uint2 u[2];                                   // value 16 nt + l % 16, rows 16 w + 4 (l / 16) ..
+    f32x4 e[2];                                   // keys 32 w + 16 mt + 4 (l / 16) ..
+};
+
 // Pass 2: one head's NV value columns of one request through the chunks of the pass, in order. The state
 // S[128 keys][NV] lives in MFMA accumulators: wave w owns keys 32 w .. 32 w + 31.
 template <typename S>
-__global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) inter_kernel(
+__global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 2))) inter_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
         const S* state_in, S* state_out, const long long* __restrict__ state_off,
         bf16_t* __restrict__ out, long long out_stride, const unsigned char* __restrict__ ws) {
@@ -673,54 +677,39 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         }
 
     const unsigned char* wsh = ws + ((long long)b * H + h) * chunks * (long long)WS_BYTES;
-    // Staging of a chunk's workspace: global -> registers -> LDS, two chunks deep at both levels. While chunk c is
-    // computed from LDS buffer c % 2, chunk c + 1 moves from its registers into the other buffer and chunk c + 2
-    // is requested into the registers chunk c came from. Every piece index q has its own array element, so source
-    // and destination are compile-time functions of q: W (q 0-3), Qg (4-7), Kg^T (8-11), M (12-13), this block's
-    // rows of U^T (14), e^{G_last} (15, 32 lanes).
-    static_assert(STAGE_PER_LANE == 16 && NV == 32, "staging map");
-    u32x4 stage_a[STAGE_PER_LANE], stage_b[STAGE_PER_LANE];
-    const unsigned stage_lo = (unsigned)t * 16u;
-    // The sixteen loads of a chunk go out in four groups spread over a chunk's phases (PART_ 0..3: W, Qg, Kg^T, the
-    // rest): sixty-four kilobytes per workgroup take the vector memory pipeline longer to accept than a phase
-    // lasts, and a wave that issues them back to back stalls on the full queue.
-#define KDA_STAGE_LOAD(ST_, C_, PART_)                                                                              \
+    // Per-lane byte offsets of the fragments inside a chunk's workspace.
+    const unsigned off_a = (unsigned)(((SUB * wave + cl) * 32 + 8 * (lane >> 4)) * 2);   // W, Qg, M: + 4096 ks
+    const unsigned off_k = (unsigned)(WS_KGT + ((32 * wave + cl) * 32 + 8 * (lane >> 4)) * 2);  // + 1024 mt + 8192 ks
+    const unsigned off_u = (unsigned)(WS_UT + ((NV * vb + cl) * CH + SUB * wave + rl) * 2);     // + 2048 nt
+    const unsigned off_e = (unsigned)(WS_E + (32 * wave + rl) * 4);                             // + 64 mt
+    // The loads of chunk C_ into operand set X_, one group at a time (each group is requested as soon as the
+    // chunk two before it has used those registers). Unconditional: past the end they repeat the last chunk.
+#define KDA_LOAD_W(X_, C_)                                                                                          \
     {                                                                                                               \
         const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                               \
-        if ((PART_) == 0) {                                                                                         \
-            _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                           \
-                ST_[q] = *reinterpret_cast<const u32x4*>(src_ + WS_W + q * 4096 + stage_lo);                         \
-        } else if ((PART_) == 1) {                                                                                  \
-            _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                           \
-                ST_[4 + q] = *reinterpret_cast<const u32x4*>(src_ + WS_QG + q * 4096 + stage_lo);                    \
-        } else if ((PART_) == 2) {                                                                                  \
-            _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                           \
-                ST_[8 + q] = *reinterpret_cast<const u32x4*>(src_ + WS_KGT + q * 4096 + stage_lo);                   \
-        } else {                                                                                                    \
-            ST_[12] = *reinterpret_cast<const u32x4*>(src_ + WS_M + stage_lo);                                      \
-            ST_[13] = *reinterpret_cast<const u32x4*>(src_ + WS_M + 4096 + stage_lo);                               \
-            ST_[14] = *reinterpret_cast<const u32x4*>(src_ + WS_UT + NV * vb * CH * 2 + stage_lo);                  \
-            ST_[15] = *reinterpret_cast<const u32x4*>(src_ + WS_E + (stage_lo & 511u));                             \
-        }                                                                                                           \
+        _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                            \
+            X_.w[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_W + off_a + 4096 * ks);                              \
+        _Pragma("unroll") for (int nt = 0; nt < 2; ++nt)                                                            \
+            X_.u[nt] = *reinterpret_cast<const uint2*>(src_ + off_u + 2048 * nt);                                    \
     }
-#define KDA_STAGE_LOAD_ALL(ST_, C_)                                                                                 \
-    KDA_STAGE_LOAD(ST_, C_, 0) KDA_STAGE_LOAD(ST_, C_, 1) KDA_STAGE_LOAD(ST_, C_, 2) KDA_STAGE_LOAD(ST_, C_, 3)
-    // 128-wide rows take 16 pieces each, 64-wide rows 8
-#define KDA_STAGE_STORE(ST_, BUF_)                                                                                  \
+#define KDA_LOAD_QM(X_, C_)                                                                                         \
     {                                                                                                               \
-        unsigned char* buf_ = smem + (BUF_) * N_BUF;                                                                \
-        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                                             \
-            const int v_ = q * THREADS + t;                                                                         \
-            *reinterpret_cast<u32x4*>(buf_ + N_W + ((v_ >> 4) * LD128 + (v_ & 15) * 8) * 2) = ST_[q];                \
-            *reinterpret_cast<u32x4*>(buf_ + N_Q + ((v_ >> 4) * LD128 + (v_ & 15) * 8) * 2) = ST_[4 + q];            \
-            *reinterpret_cast<u32x4*>(buf_ + N_K + ((v_ >> 3) * LD64 + (v_ & 7) * 8) * 2) = ST_[8 + q];              \
-        }                                                                                                           \
-        *reinterpret_cast<u32x4*>(buf_ + N_M + ((t >> 3) * LD64 + (t & 7) * 8) * 2) = ST_[12];                      \
-        *reinterpret_cast<u32x4*>(buf_ + N_M + (((THREADS + t) >> 3) * LD64 + (t & 7) * 8) * 2) = ST_[13];          \
-        *reinterpret_cast<u32x4*>(buf_ + N_U + ((t >> 3) * LD64 + (t & 7) * 8) * 2) = ST_[14];                      \
-        if (t < 32) *reinterpret_cast<u32x4*>(buf_ + N_E + t * 16) = ST_[15];                                       \
+        const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                               \
+        _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                            \
+            X_.q[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_QG + off_a + 4096 * ks);                             \
+        _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                            \
+            X_.m[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_M + off_a + 4096 * ks);                              \
     }
-    // S^T for the first chunk
+#define KDA_LOAD_KE(X_, C_)                                                                                         \
+    {                                                                                                               \
+        const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                               \
+        _Pragma("unroll") for (int mt = 0; mt < 2; ++mt) {                                                          \
+            _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                        \
+                X_.k[mt][ks] = *reinterpret_cast<const u32x4*>(src_ + off_k + 1024 * mt + 8192 * ks);                \
+            X_.e[mt] = *reinterpret_cast<const f32x4*>(src_ + off_e + 64 * mt);                                      \
+        }                                                                                                           \
+    }
+    // S^T (fp16) for the products of a chunk
     auto put_state = [&]() {
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -731,25 +720,14 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
                 *reinterpret_cast<uint2*>(Sl + (SUB * nt + cl) * LD128 + 32 * wave + SUB * mt + rl) = make_uint2(s0, s1);
             }
     };
+    auto as_u4 = [](const u32x4 v) { return make_uint4(v[0], v[1], v[2], v[3]); };
 
-    // Chunk c from LDS buffer `buf`. `mine` are the registers its workspace came through: free now, they take
-    // chunk c + 2; `next` hold chunk c + 1, which goes to the other buffer. Both moves are unconditional (past the
-    // end they repeat the last chunk, unused), so that the wait for `next` can be counted in loads still in flight.
-    auto chunk_step = [&](const int c, const int buf, u32x4 (&mine)[STAGE_PER_LANE], u32x4 (&next)[STAGE_PER_LANE])
-                          __attribute__((always_inline)) {
+    // Chunk c with the operands in x; each group of x is then requested again for chunk c + 2.
+    auto chunk_step = [&](const int c, InterOperands& x) __attribute__((always_inline)) {
         const int nrows = min(CH, left - c * CH);
-        const uint16_t* Wl = reinterpret_cast<const uint16_t*>(smem + buf * N_BUF + N_W);
-        const uint16_t* Ql = reinterpret_cast<const uint16_t*>(smem + buf * N_BUF + N_Q);
-        const uint16_t* Kl = reinterpret_cast<const uint16_t*>(smem + buf * N_BUF + N_K);
-        const uint16_t* Ml = reinterpret_cast<const uint16_t*>(smem + buf * N_BUF + N_M);
-        const uint16_t* Ul = reinterpret_cast<const uint16_t*>(smem + buf * N_BUF + N_U);
-        const float* El = reinterpret_cast<const float*>(smem + buf * N_BUF + N_E);
-        put_state();
-        __syncthreads();      // the state and (stored during the chunk before) this chunk's workspace are in LDS;
-                              // every wave is done with the chunk before, so the other buffer, S and V' are free
         const int c2 = min(c + 2, nch - 1);
-        KDA_STAGE_STORE(next, 1 - buf)
-        KDA_STAGE_LOAD(mine, c2, 0)
+        put_state();
+        __syncthreads();      // the state is in LDS; every wave is done with the V' of the chunk before
         const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
         // V' = U - W S: wave w takes rows 16 w .. 16 w + 15
         uint4 sfrag[2][4];
@@ -757,23 +735,21 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) sfrag[nt][ks] = frag(Sl, LD128, SUB * nt, 32 * ks, lane);
-        KDA_STAGE_LOAD(mine, c2, 1)
         f32x4 accV[2] = {zero, zero};
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const uint4 a = frag(Wl, LD128, SUB * wave, 32 * ks, lane);
+        for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt) accV[nt] = mfma_f16(a, sfrag[nt][ks], accV[nt]);
-        }
+            for (int nt = 0; nt < 2; ++nt) accV[nt] = mfma_f16(as_u4(x.w[ks]), sfrag[nt][ks], accV[nt]);
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt) {
-            const uint2 u = *reinterpret_cast<const uint2*>(Ul + (SUB * nt + cl) * LD64 + SUB * wave + rl);
+            const uint2 u = x.u[nt];
             const float v0 = h2f((uint16_t)(u.x & 0xffffu)) - accV[nt][0], v1 = h2f((uint16_t)(u.x >> 16)) - accV[nt][1];
             const float v2 = h2f((uint16_t)(u.y & 0xffffu)) - accV[nt][2], v3 = h2f((uint16_t)(u.y >> 16)) - accV[nt][3];
             const uint32_t p0 = (uint32_t)f2h(v0) | ((uint32_t)f2h(v1) << 16);
             const uint32_t p1 = (uint32_t)f2h(v2) | ((uint32_t)f2h(v3) << 16);
             *reinterpret_cast<uint2*>(Vl + (SUB * nt + cl) * LD64 + SUB * wave + rl) = make_uint2(p0, p1);
         }
+        KDA_LOAD_W(x, c2)
         __syncthreads();
         // Y = Qg S + M V'
         uint4 vfrag[2][2];
@@ -781,21 +757,16 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) vfrag[nt][ks] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
-        KDA_STAGE_LOAD(mine, c2, 2)
         f32x4 accY[2] = {zero, zero};
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const uint4 a = frag(Ql, LD128, SUB * wave, 32 * ks, lane);
+        for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt) accY[nt] = mfma_f16(a, sfrag[nt][ks], accY[nt]);
-        }
+            for (int nt = 0; nt < 2; ++nt) accY[nt] = mfma_f16(as_u4(x.q[ks]), sfrag[nt][ks], accY[nt]);
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            const uint4 a = frag(Ml, LD64, SUB * wave, 32 * ks, lane);
+        for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt) accY[nt] = mfma_f16(a, vfrag[nt][ks], accY[nt]);
-        }
-        KDA_STAGE_LOAD(mine, c2, 3)
+            for (int nt = 0; nt < 2; ++nt) accY[nt] = mfma_f16(as_u4(x.m[ks]), vfrag[nt][ks], accY[nt]);
+        KDA_LOAD_QM(x, c2)
         {
             const long long grow0 = rr.row0 + sub0 + c * CH;
 #pragma unroll
@@ -810,19 +781,16 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         // S <- e^{G_last} S + Kg^T V'
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
-            const float4 e = *reinterpret_cast<const float4*>(El + 32 * wave + SUB * mt + rl);
-            const float ev[4] = {e.x, e.y, e.z, e.w};
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) accS[mt][nt][r] *= ev[r];
+                for (int r = 0; r < 4; ++r) accS[mt][nt][r] *= x.e[mt][r];
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                const uint4 a = frag(Kl, LD64, 32 * wave + SUB * mt, 32 * ks, lane);
+            for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                for (int nt = 0; nt < 2; ++nt) accS[mt][nt] = mfma_f16(a, vfrag[nt][ks], accS[mt][nt]);
-            }
+                for (int nt = 0; nt < 2; ++nt) accS[mt][nt] = mfma_f16(as_u4(x.k[mt][ks]), vfrag[nt][ks], accS[mt][nt]);
         }
+        KDA_LOAD_KE(x, c2)
         if constexpr (sizeof(S) == 2) {
             // a bf16 state is rounded at the end of every chunk, so the result does not depend on where passes end
 #pragma unroll
@@ -834,17 +802,18 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         }
     };
     if (nch > 0) {
-        KDA_STAGE_LOAD_ALL(stage_a, 0)
-        KDA_STAGE_LOAD_ALL(stage_b, min(1, nch - 1))
-        KDA_STAGE_STORE(stage_a, 0)
-        // in pairs, so that the register sets and LDS buffers are compile-time choices; an odd last chunk follows
+        InterOperands xa, xb;                     // even and odd chunks
+        KDA_LOAD_W(xa, 0) KDA_LOAD_QM(xa, 0) KDA_LOAD_KE(xa, 0)
+        const int c1 = min(1, nch - 1);
+        KDA_LOAD_W(xb, c1) KDA_LOAD_QM(xb, c1) KDA_LOAD_KE(xb, c1)
+        // in pairs, so that the operand sets are compile-time choices; an odd last chunk follows
         int c = 0;
 #pragma unroll 1
         for (; c + 1 < nch; c += 2) {
-            chunk_step(c, 0, stage_a, stage_b);
-            chunk_step(c + 1, 1, stage_b, stage_a);
+            chunk_step(c, xa);
+            chunk_step(c + 1, xb);
         }
-        if (c < nch) chunk_step(c, 0, stage_a, stage_b);
+        if (c < nch) chunk_step(c, xa);
     }
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
