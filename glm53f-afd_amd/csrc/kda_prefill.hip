@@ -494,7 +494,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
     // M and -L above the block diagonal are zero: blocks (0,1), (0,2), (0,3), (1,2), (1,3), (2,3)
     {
         uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
-        for (int e = t; e < 6 * 256; e += THREADS) {
+        // by waves 1 to 3: wave 0 goes straight to the inversion below
+        for (int e = t - 64; e >= 0 && e < 6 * 256; e += THREADS - 64) {
             const int blk = e >> 8, r = (e >> 4) & 15, cc = e & 15;
             const int rb = blk < 3 ? 0 : (blk < 5 ? 1 : 2);
             const int cb = blk < 3 ? blk + 1 : (blk < 5 ? blk - 1 : 3);
@@ -509,13 +510,28 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
     if (t < CH) {
         const int a = t >> 4, j = t & 15;
         const float bj = beta_s[t];
-        float x[SUB];
+        // the block's strictly lower triangle into registers (rows as 128-bit pieces), then the substitution
+        // column by column: once x[m] is known every later row takes its term, sixteen independent chains
+        float l[SUB][SUB];
+#pragma unroll
+        for (int i = 1; i < SUB; ++i)
+#pragma unroll
+            for (int p = 0; p < (i + 3) / 4; ++p) {
+                const f32x4 v = *reinterpret_cast<const f32x4*>(Ld + (SUB * a + i) * LDD + 4 * p);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) l[i][4 * p + e] = v[e];
+            }
+        float acc[SUB], x[SUB];
+#pragma unroll
+        for (int i = 0; i < SUB; ++i) acc[i] = 0.0f;
+#pragma unroll
+        for (int m = 0; m < SUB; ++m) {
+            x[m] = m < j ? 0.0f : (m == j ? 1.0f : -acc[m]);
+#pragma unroll
+            for (int i = m + 1; i < SUB; ++i) acc[i] = __builtin_fmaf(l[i][m], x[m], acc[i]);
+        }
 #pragma unroll
         for (int i = 0; i < SUB; ++i) {
-            float acc = 0.0f;
-#pragma unroll
-            for (int m = 0; m < i; ++m) acc = __builtin_fmaf(Ld[(SUB * a + i) * LDD + m], x[m], acc);
-            x[i] = i < j ? 0.0f : (i == j ? 1.0f : -acc);
             TT[(SUB * a + i) * LDT + j] = f2h(x[i] * bj);
             TT[(SUB * a + i) * LDT + SUB + j] = f2h(x[i]);
         }
