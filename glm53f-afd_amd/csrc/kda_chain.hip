@@ -280,21 +280,39 @@ __global__ void conv_shift_kernel(int C, const int32_t* __restrict__ cu_rows, co
                                   int keep1, bf16_t* conv, long long conv_stride,
                                   const long long* __restrict__ conv_off, const bf16_t* P,
                                   long long p_layer_stride, long long p_stride) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= C) return;
     const int layer = blockIdx.y, b = blockIdx.z;
     const long long row0 = cu_rows != nullptr ? cu_rows[b] : 0;
     const int k = keep != nullptr ? keep[b] : keep1;
     bf16_t* win = conv + (long long)layer * conv_stride + (conv_off != nullptr ? conv_off[b] : 0);
     const bf16_t* rows = P + (long long)layer * p_layer_stride + row0 * p_stride;
-    bf16_t v[WINDOW];
+    // Eight channels per lane in 128-bit pieces when every row involved is 16-byte aligned (uniform over the
+    // workgroup), else one channel per lane; the grid covers C channels either way (see the launcher).
+    const bool wide = (C % 8 == 0) && (p_stride % 8 == 0) &&
+                      ((reinterpret_cast<uintptr_t>(win) | reinterpret_cast<uintptr_t>(rows)) & 15u) == 0;
+    if (wide) {
+        const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+        if (c >= C) return;
+        uint4 v[WINDOW];
 #pragma unroll
-    for (int j = 0; j < WINDOW; ++j) {
-        const long long src = (long long)k + j;
-        v[j] = src < WINDOW ? win[src * C + c] : rows[(src - WINDOW) * p_stride + c];
+        for (int j = 0; j < WINDOW; ++j) {
+            const long long src = (long long)k + j;
+            v[j] = ld128(src < WINDOW ? win + src * C + c : rows + (src - WINDOW) * p_stride + c);
+        }
+#pragma unroll
+        for (int j = 0; j < WINDOW; ++j) st128(win + (long long)j * C + c, v[j]);
+        return;
     }
+    for (int c = blockIdx.x * blockDim.x * 8 + threadIdx.x; c < min(C, (int)(blockIdx.x + 1) * (int)blockDim.x * 8);
+         c += blockDim.x) {
+        bf16_t v[WINDOW];
 #pragma unroll
-    for (int j = 0; j < WINDOW; ++j) win[(long long)j * C + c] = v[j];
+        for (int j = 0; j < WINDOW; ++j) {
+            const long long src = (long long)k + j;
+            v[j] = src < WINDOW ? win[src * C + c] : rows[(src - WINDOW) * p_stride + c];
+        }
+#pragma unroll
+        for (int j = 0; j < WINDOW; ++j) win[(long long)j * C + c] = v[j];
+    }
 }
 
 // Commit by selection: workgroup (layer * H + h, b) copies one head of the checkpoint after row keep[b] - 1.
@@ -383,7 +401,7 @@ inline int conv_shift_launch(int32_t channels, int32_t layers, int32_t batch, co
                              glm53f_stream_t stream) {
     if (channels < 1 || layers < 1 || layers > 65535 || batch < 1 || batch > 65535 || !conv || !p || keep1 < 0)
         return kInvalid;
-    const dim3 grid((channels + kShiftThreads - 1) / kShiftThreads, layers, batch);
+    const dim3 grid((channels + 8 * kShiftThreads - 1) / (8 * kShiftThreads), layers, batch);   // 8 channels per lane
     conv_shift_kernel<<<grid, kShiftThreads, 0, (hipStream_t)stream>>>(
         channels, cu_rows, keep, keep1, bfp(conv), conv_stride, reinterpret_cast<const long long*>(conv_off), bfp(p),
         p_layer_stride, p_stride);

@@ -384,3 +384,30 @@ def test_bad_arguments_are_rejected():
                                            hs.ptr(conv_d), 0, hs.ptr(meta.conv_off), hs.ptr(sr.p), 0, sr.p_stride,
                                            None) == 1
     hs.sync()
+
+
+def test_conv_shift_wide_and_narrow_paths_agree_with_the_oracle():
+    """The shift moves eight channels per lane when every row is 16-byte aligned and one channel per lane
+    otherwise (rows starting at an odd element, a channel count that is no multiple of eight): same bits."""
+    heads = 4
+    c = channels(heads)
+    rows = o.synth_rows(heads, 5, 910)
+    conv = o.synth_conv_window(heads, 911)
+    qkv = rows.qkv.reshape(5, c)
+    for keep in (0, 1, 2, 3, 5):
+        want = o.conv_shift(conv, rows, keep)
+        for shift, stride in ((0, c), (1, c + 8), (3, c + 5)):
+            p = torch.zeros(5 * stride + 8, dtype=torch.bfloat16, device=hs.DEV)
+            p[shift:shift + 5 * stride].view(5, stride)[:, :c] = hs.to_bf16(qkv)
+            conv_d = hs.to_bf16(conv)
+            hs.check(ffi.glm53f_kda_conv_shift(c, keep, hs.ptr(conv_d), hs.ptr(p, shift), stride, None), "conv shift")
+            hs.sync()
+            assert np.array_equal(hs.back(conv_d), want), (keep, shift, stride)
+    # a channel count that is not a multiple of eight (the kernel takes any count)
+    cc = c - 3
+    win = torch.arange(3 * cc, device=hs.DEV).to(torch.bfloat16)
+    p = (1000 + torch.arange(2 * cc, device=hs.DEV)).to(torch.bfloat16)
+    before = win.clone()
+    hs.check(ffi.glm53f_kda_conv_shift(cc, 2, hs.ptr(win), hs.ptr(p), cc, None), "conv shift")
+    hs.sync()
+    assert torch.equal(win.view(3, cc), torch.cat([before.view(3, cc)[2:], p.view(2, cc)]))
