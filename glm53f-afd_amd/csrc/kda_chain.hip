@@ -78,46 +78,101 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
     }
     const float decay_rate = expf(a_log[h]);
 
-    // A row's prologue. Every global load of the row goes out first, back to back and without branches (lanes
-    // that have no use for a value load a neighbour's and drop it), so a row pays one memory latency, not one
-    // per stage: the inputs and weights of conv channel t of q|k (q for t < 128, k after) and of v channel
-    // t % 128, the forget-gate input and bias of key channel t % 128, the beta logit, and the output gate and
-    // norm weight of value channel t % 128 for the row's epilogue.
-    const int i7 = t & (DK - 1);
-    const unsigned c0 = (unsigned)((t >> 7) * H * DK + h * DK + i7);      // q | k channel of this lane
-    const unsigned c1 = (unsigned)(2 * H * DK + h * DK + i7);             // v channel (lanes 0..127 use it)
-    float gate_r = 0.0f, normw_r = 0.0f;                                  // the epilogue's operands
-    struct RowIn {
-        uint2 w0, w1;
-        bf16_t x0[TAPS], x1[TAPS];
-        bf16_t a_raw, b_raw, g_raw, nw_raw;
-        float dtb;
+    // Inputs reach the workgroup as 128-bit pieces, one per lane, staged in LDS: per-lane 16-bit loads would take
+    // seventeen memory instructions per lane and row, and sixteen waves a CU issuing those keep its address
+    // pipeline busy for microseconds before the state's loads can even start.
+    //   weights, once: conv weights of the head's 384 channels (pieces 0..191), dt_bias (192..223), norm weight
+    //   (224..239);  a row: its four conv taps of q | k | v (pieces 0..191, tap-major), its forget-gate inputs
+    //   (192..207) and output-gate logits (208..223). Piece i lands at byte 16 i of its staging array.
+    __shared__ __align__(16) unsigned char w_stage[240 * 16];
+    __shared__ __align__(16) unsigned char x_stage[224 * 16];
+    const bf16_t* xs = reinterpret_cast<const bf16_t*>(x_stage);              // [4 taps][q | k | v][128]
+    const bf16_t* a_sh = xs + TAPS * 3 * DK;                                  // [128]
+    const bf16_t* gate_sh = a_sh + DK;                                        // [128]
+    // 16 bytes from an address with 2-byte alignment or better
+    auto load_piece = [](const void* p) -> u32x4_t {
+        if ((reinterpret_cast<uintptr_t>(p) & 15u) == 0) return *reinterpret_cast<const u32x4_t*>(p);
+        const uint16_t* q = reinterpret_cast<const uint16_t*>(p);
+        u32x4_t v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (uint32_t)q[2 * e] | ((uint32_t)q[2 * e + 1] << 16);
+        return v;
     };
-    auto load_row = [&](int r, RowIn& in) {
+    auto weight_piece = [&]() -> u32x4_t {
+        const int i = min(t, 239);
+        const void* p;
+        if (i < 192) p = cw + ((size_t)(i >> 6) * H * DK + (size_t)h * DK) * TAPS + (i & 63) * 8;
+        else if (i < 224) p = dt_bias + h * DK + (i - 192) * 4;
+        else p = norm_w + (i - 224) * 8;
+        return load_piece(p);
+    };
+    auto row_piece = [&](int r) -> u32x4_t {
         const long long gr = rr.row0 + r;
-        in.w0 = *reinterpret_cast<const uint2*>(cw + (size_t)c0 * TAPS);
-        in.w1 = *reinterpret_cast<const uint2*>(cw + (size_t)c1 * TAPS);
+        const int i = min(t, 223);
+        const bf16_t* p;
+        if (i < 192) {
+            const int j = i / 48, rem = i - 48 * j, at = r + j;
+            const bf16_t* row = at < WINDOW ? cs + (long long)at * C : P + (rr.row0 + at - WINDOW) * p_stride;
+            p = row + (long long)(rem >> 4) * H * DK + h * DK + (rem & 15) * 8;
+        } else if (i < 208) {
+            p = A + gr * a_stride + h * DK + (i - 192) * 8;
+        } else {
+            p = G + gr * g_stride + h * DV + (i - 208) * 8;
+        }
+        return load_piece(p);
+    };
+    auto beta_logit = [&](int r) -> bf16_t { return *uniform_ptr(P + (rr.row0 + r) * p_stride + b_off + h); };
+
+    // The first row's inputs and the weights are requested before the state (the scheduling barriers keep that
+    // order), so the prologue waits for them alone and runs while the state streams in. Between rows the state
+    // stays in its stored form (`raw`: packed bf16 pairs, or f32 bits): a bf16 state is rounded after every row
+    // anyway, and the packed form halves the registers it holds. With a bf16 state there are registers to spare and
+    // the next row's piece is requested before this row's update; an f32 state requests it after the epilogue.
+    constexpr bool kPrefetch = M::kRound;
+    const int i7 = t & (DK - 1);
+    uint4 raw[M::STEPS];
+    u32x4_t xpiece = row_piece(0);
+    bf16_t b_raw = beta_logit(0);
+    {
+        const u32x4_t wpiece = weight_piece();
+        __builtin_amdgcn_sched_barrier(0);
+        load_state<S>(state_in + sbase, soff_lane, raw);
+        __builtin_amdgcn_sched_barrier(0);
+        if (t < 240) *reinterpret_cast<u32x4_t*>(w_stage + t * 16) = wpiece;
+    }
+    __syncthreads();
+    // This lane's weights: conv channel t of q | k, v channel t % 128, the forget-gate bias of key t % 128 and the
+    // norm weight of value t % 128. They stay staged for all rows; with a bf16 state there are registers to keep
+    // them in, an f32 state reads them again for every row.
+    struct LaneWeights {
+        uint2 w0, w1;
+        float dtb, normw;
+    };
+    auto lane_weights = [&]() -> LaneWeights {
+        return {*reinterpret_cast<const uint2*>(w_stage + t * 8), *reinterpret_cast<const uint2*>(w_stage + (2 * DK + i7) * 8),
+                *reinterpret_cast<const float*>(w_stage + 192 * 16 + i7 * 4),
+                bf2f(*reinterpret_cast<const bf16_t*>(w_stage + 224 * 16 + i7 * 2))};
+    };
+    LaneWeights kept = {};
+    if constexpr (kPrefetch) kept = lane_weights();
+    float gate_r = 0.0f, normw_r = 0.0f;                                      // the epilogue's operands
+
+    // A row's prologue from its staged piece: conv + SiLU, gates, L2 norms.
+    auto prologue = [&]() {
+        if (t < 224) *reinterpret_cast<u32x4_t*>(x_stage + t * 16) = xpiece;
+        __syncthreads();
+        bf16_t x0[TAPS], x1[TAPS];
 #pragma unroll
         for (int tap = 0; tap < TAPS; ++tap) {
-            const int at = r + tap;
-            const bf16_t* src = uniform_ptr(at < WINDOW ? cs + (long long)at * C : P + (rr.row0 + at - WINDOW) * p_stride);
-            in.x0[tap] = src[c0];
-            in.x1[tap] = src[c1];
+            x0[tap] = xs[tap * 3 * DK + t];                 // q channel t, or k channel t - 128
+            x1[tap] = xs[tap * 3 * DK + 2 * DK + i7];
         }
-        in.a_raw = uniform_ptr(A + gr * a_stride + h * DK)[(unsigned)i7];
-        in.dtb = (dt_bias + h * DK)[(unsigned)i7];
-        in.b_raw = *uniform_ptr(P + gr * p_stride + b_off + h);
-        in.g_raw = uniform_ptr(G + gr * g_stride + h * DV)[(unsigned)i7];
-        in.nw_raw = norm_w[i7];
-    };
-    auto prologue = [&](const RowIn& in) {
-        const uint2 w0 = in.w0, w1 = in.w1;
-        const bf16_t (&x0)[TAPS] = in.x0;
-        const bf16_t (&x1)[TAPS] = in.x1;
-        const bf16_t a_raw = in.a_raw, b_raw = in.b_raw;
-        const float dtb = in.dtb;
-        gate_r = bf2f(in.g_raw);
-        normw_r = bf2f(in.nw_raw);
+        const bf16_t a_raw = a_sh[i7];
+        gate_r = bf2f(gate_sh[i7]);
+        const LaneWeights lw = kPrefetch ? kept : lane_weights();
+        const uint2 w0 = lw.w0, w1 = lw.w1;
+        const float dtb = lw.dtb;
+        normw_r = lw.normw;
         // conv + SiLU, one bf16 rounding (cpu.rs:257-281)
         auto conv1 = [&](const uint2 w4, const bf16_t (&x)[TAPS]) -> float {
             const float wt[TAPS] = {__uint_as_float(w4.x << 16), __uint_as_float(w4.x & 0xffff0000u),
@@ -152,24 +207,15 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
         __syncthreads();
     };
 
-    // The first row's inputs are requested before the state (the scheduling barriers keep that order), so the
-    // prologue waits for them alone and runs while the state streams in. Between rows the state stays in its
-    // stored form (`raw`: packed bf16 pairs, or f32 bits): a bf16 state is rounded after every row anyway, and
-    // the packed form halves the registers it holds. With a bf16 state there are registers to spare, and the
-    // next row's inputs are requested before this row's update; an f32 state requests them after the epilogue.
-    constexpr bool kPrefetch = M::kRound;
-    uint4 raw[M::STEPS];
-    RowIn in;
-    load_row(0, in);
-    __builtin_amdgcn_sched_barrier(0);
-    load_state<S>(state_in + sbase, soff_lane, raw);
-    __builtin_amdgcn_sched_barrier(0);
     int r = 0;
     do {   // rows >= 1 here; a do-while leaves no zero-trip path that would keep the loaded state alive
         const long long gr = rr.row0 + r;
-        prologue(in);
+        prologue();
         if constexpr (kPrefetch) {
-            if (r + 1 < rows) load_row(r + 1, in);
+            if (r + 1 < rows) {
+                xpiece = row_piece(r + 1);
+                b_raw = beta_logit(r + 1);
+            }
         }
         const float beta = beta_s;
         // Stores leave as soon as a step's 16 or 8 value rows are final, so they overlap the remaining steps
@@ -220,7 +266,10 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
         }
         __syncthreads();
         if constexpr (!kPrefetch) {
-            if (r + 1 < rows) load_row(r + 1, in);
+            if (r + 1 < rows) {
+                xpiece = row_piece(r + 1);
+                b_raw = beta_logit(r + 1);
+            }
         }
     } while (++r < rows);
 }

@@ -13,6 +13,7 @@ constexpr int DK = 128, DV = 128, TAPS = 4, WINDOW = 3;
 constexpr int kInvalid = 1;  // hipErrorInvalidValue
 
 typedef uint16_t bf16_t;
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));   // a 128-bit piece that stays in registers
 
 __device__ __forceinline__ float bf2f(bf16_t b) { return __uint_as_float((uint32_t)b << 16); }
 
