@@ -33,9 +33,9 @@ from glm53f_kda import DK, DV, HEADS, LAYERS, WINDOW, channels, ffi, state_len
 # script's legs, scaled by the same counters over the 1 GiB copy of --only copy: x2.00 and x1.00). Measured
 # offline; the summaries are kept in profiles/.
 TRAFFIC_BYTES = {
-    "decode_chain": (36_792 + 33_024) * 1024,            # per chain launch, 16 slots x 1 row
-    "verify_chain": (223_800 + 1_585_152) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
-    "prefill_2048_rows": (139_573 + 149_043 + 152_661 + 36_864 + 65_580 + 32_768 + 172 + 144) * 1024,
+    "decode_chain": (36_805 + 33_024) * 1024,            # per chain launch, 16 slots x 1 row
+    "verify_chain": (226_538 + 1_585_152) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
+    "prefill_2048_rows": (135_598 + 148_845 + 152_700 + 36_864 + 65_571 + 32_768 + 172 + 144) * 1024,
 }
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
