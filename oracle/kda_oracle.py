@@ -89,6 +89,7 @@ def _declare(l: C.CDLL) -> None:
         "kda_gated_rmsnorm_as": (None, [vp, vp, vp, f32, C.c_int, vp]),
         "kda_chain_with": (None, [vp, vp, vp, vp, C.c_int, C.c_int, vp, vp, vp, vp, vp, vp, vp, C.c_int]),
         "kda_replay_with": (None, [i32, vp, vp, vp, vp, vp, i32, C.c_int, vp]),
+        "kda_exact_replay": (None, [i32, vp, vp, vp, vp, vp, i32, vp, C.c_int]),
         "kda_conv_shift": (None, [i32, vp, vp, i32, i32, vp]),
         "kda_transpose_state": (None, [vp, vp, i64]),
         "kda_literal_l2norm": (None, [vp, vp]),
@@ -113,7 +114,7 @@ EXPORTS = [
     "kda_rng_fill", "kda_rng_fill_bf16", "kda_rng_normal", "kda_rng_fill_normal", "kda_synth_layer",
     "kda_synth_rows", "kda_synth_conv_window", "kda_synth_state", "kda_sigmoid", "kda_silu", "kda_warp_sum",
     "kda_dot128", "kda_log_decay", "kda_decay", "kda_beta", "kda_q_scale", "kda_conv_channel", "kda_conv_qkv",
-    "kda_l2norm", "kda_update", "kda_read_out", "kda_gated_rmsnorm_as", "kda_chain_with", "kda_replay_with",
+    "kda_l2norm", "kda_update", "kda_read_out", "kda_gated_rmsnorm_as", "kda_chain_with", "kda_replay_with", "kda_exact_replay",
     "kda_conv_shift", "kda_transpose_state", "kda_literal_l2norm", "kda_literal_step",
     "kda_literal_gated_rmsnorm_as", "kda_literal_chain", "kda_chunked_head", "kda_chunked_layer",
     "kda_recurrent_layer", "kda_prefill_head", "kda_prefill",
@@ -411,6 +412,18 @@ def replay(state, saves: Saves, keep: int, bf16_state: bool = False) -> np.ndarr
     out = np.empty_like(state)
     k, v, g, b = _f32(saves.k), _f32(saves.v), _f32(saves.g), _f32(saves.beta)
     lib().kda_replay_with(saves.heads, _p(state), _p(k), _p(v), _p(g), _p(b), keep, int(bf16_state), _p(out))
+    return out
+
+
+def exact_replay(state, saves: Saves, rows: int | None = None, threads: int = 1) -> np.ndarray:
+    """The delta rule over the saved rows in f64 (tests/gpu_prefill.rs:502-519): float64 state [H][DV][DK]."""
+    rows = saves.rows if rows is None else rows
+    assert rows <= saves.rows
+    state = _f32(state)
+    out = np.empty(state.size, dtype=np.float64)
+    k, v, g, b = _f32(saves.k), _f32(saves.v), _f32(saves.g), _f32(saves.beta)
+    lib().kda_exact_replay(saves.heads, _p(state), _p(k), _p(v), _p(g), _p(b), rows, out.ctypes.data_as(C.c_void_p),
+                           threads)
     return out
 
 

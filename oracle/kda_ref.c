@@ -297,6 +297,30 @@ void kda_replay_with(int32_t heads, const float* state, const float* k_save, con
     }
 }
 
+/* tests/gpu_prefill.rs:502-519 */
+void kda_exact_replay(int32_t heads, const float* state, const float* k_save, const float* v_save,
+                      const float* g_save, const float* b_save, int32_t rows, double* state_out, int threads) {
+#pragma omp parallel for num_threads(threads > 1 ? threads : 1) schedule(dynamic)
+    for (int32_t h = 0; h < heads; ++h) {
+        double* s = state_out + (int64_t)h * DV * DK;
+        for (int i = 0; i < DV * DK; ++i) s[i] = (double)state[(int64_t)h * DV * DK + i];
+        for (int32_t r = 0; r < rows; ++r) {
+            const int64_t at = ((int64_t)r * heads + h) * DK;
+            const double beta = (double)b_save[(int64_t)r * heads + h];
+            for (int row = 0; row < DV; ++row) {
+                double* sr = s + row * DK;
+                double kv = 0.0;
+                for (int k = 0; k < DK; ++k) {
+                    sr[k] *= (double)g_save[at + k];
+                    kv += sr[k] * (double)k_save[at + k];
+                }
+                const double delta = ((double)v_save[at + row] - kv) * beta;
+                for (int k = 0; k < DK; ++k) sr[k] += (double)k_save[at + k] * delta;
+            }
+        }
+    }
+}
+
 /* cpu.rs:512-527 */
 void kda_conv_shift(int32_t heads, const float* conv, const float* qkv, int32_t rows, int32_t keep, float* out) {
     const int64_t cn = channels(heads);

@@ -14,6 +14,7 @@
  *   l2norm, gated_rmsnorm    known answers of tests/cpu_reference.rs:124-145
  *   update, read_out, chain  invariants of tests/cpu_reference.rs:148-257, an f64 textbook recurrence
  *   literal_*                tests/cpu_reference.rs:260-285, the f64 textbook recurrence
+ *   exact_replay             the same f64 recurrence written independently in the tests (numpy), small inputs
  *   chunked_head/layer       exact-arithmetic identity with the recurrence, tests/cpu_reference.rs:348-384
  *   prefill_head/prefill     tests/cpu_reference.rs:399-450
  * Bit-level agreement with the transformers 5.17.0 `chunk_kimi_delta_attention` on real activations is
@@ -117,6 +118,10 @@ void kda_chain_with(const kda_layer* p, const float* conv, const float* state, c
                     float* g_save, float* b_save, int threads);
 void kda_replay_with(int32_t heads, const float* state, const float* k_save, const float* v_save,
                      const float* g_save, const float* b_save, int32_t keep, int bf16_state, float* state_out);
+/* The delta rule over saved rows in f64, from an f32 state: the exact-arithmetic yardstick of the reference's
+ * accuracy tests (tests/gpu_prefill.rs:502-519, tests/gpu_bf16_state.rs:660-682). Heads run in parallel. */
+void kda_exact_replay(int32_t heads, const float* state, const float* k_save, const float* v_save,
+                      const float* g_save, const float* b_save, int32_t rows, double* state_out, int threads);
 void kda_conv_shift(int32_t heads, const float* conv, const float* qkv, int32_t rows, int32_t keep, float* out);
 void kda_transpose_state(const float* s, float* t, int64_t n);
 

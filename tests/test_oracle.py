@@ -479,3 +479,24 @@ def test_oracle_exports_every_declared_symbol():
     assert declared == set(o.EXPORTS)
     for name in declared:
         assert hasattr(o.lib(), name)
+
+
+def test_exact_replay_is_the_f64_recurrence():
+    """The f64 yardstick of the accuracy tests against the same recurrence written with numpy."""
+    heads, n = 2, 6
+    p, conv, s0 = o.synth_layer(heads, 5), o.synth_conv_window(heads, 5), o.synth_state(heads, 5, 0.5)
+    c = o.chain(p, conv, s0, o.synth_rows(heads, n, 5))
+    got = o.exact_replay(s0, c.saves).reshape(heads, 128, 128)
+    s = s0.astype(np.float64).reshape(heads, 128, 128).copy()
+    k = c.saves.k.reshape(n, heads, 128).astype(np.float64)
+    v = c.saves.v.reshape(n, heads, 128).astype(np.float64)
+    g = c.saves.g.reshape(n, heads, 128).astype(np.float64)
+    b = c.saves.beta.reshape(n, heads).astype(np.float64)
+    for r in range(n):
+        for h in range(heads):
+            s[h] *= g[r, h][None, :]
+            s[h] += np.outer((v[r, h] - s[h] @ k[r, h]) * b[r, h], k[r, h])
+    assert np.max(np.abs(got - s)) <= 1e-15
+    # a prefix, and the f32 chain is within f32 rounding of it
+    assert np.array_equal(o.exact_replay(s0, c.saves, rows=0), s0.astype(np.float64))
+    assert np.max(np.abs(c.state - got.reshape(-1))) <= 1e-6 * np.max(np.abs(got))
