@@ -292,6 +292,31 @@ def bench_verify(steps, warmup, stream):
 
     ms_v = timed(verify, steps, warmup, stream)
     ms_s = timed(select, steps, warmup, stream)
+
+    # The reference's form of the same round, for comparison: the verify pass saves every row's replay inputs
+    # (1,284 B per row and head) and leaves the state alone; the commit replays the kept prefix from the saves.
+    total = slots_n * drafts
+    sk = torch.empty(layers, total * heads * DK, device=DEV)
+    sv = torch.empty(layers, total * heads * DV, device=DEV, dtype=torch.bfloat16)
+    sg = torch.empty(layers, total * heads * DK, device=DEV)
+    sb = torch.empty(layers, total * heads, device=DEV)
+    cfn, rfn = ffi.glm53f_kda_chain_batch_bf16state, ffi.glm53f_kda_replay_batch_bf16state
+    cargs = [(heads, slots_n, ptr(cu), *rows.row_args(), ptr(convs[l]), ptr(coff), ptr(layer.conv_w), ptr(pools[l]),
+              None, ptr(soff), *layer.args(), *rows.out_args(), ptr(sk[l]), ptr(sv[l]), ptr(sg[l]), ptr(sb[l]), st)
+             for l in range(layers)]
+    rargs = [(heads, 1, slots_n, ptr(cu), ptr(keep), ptr(pools[l]), ptr(pools[l]), 0, ptr(soff), ptr(sk[l]), ptr(sv[l]),
+              ptr(sg[l]), ptr(sb[l]), 0, 0, st) for l in range(layers)]
+
+    def verify_saves():
+        check(cfn(*cargs[it[0] % layers]), "chain with saves")
+        it[0] += 1
+
+    def replay():
+        check(rfn(*rargs[it[0] % layers]), "replay")
+        it[0] += 1
+
+    ms_vs = timed(verify_saves, steps, warmup, stream)
+    ms_r = timed(replay, steps, warmup, stream)
     vbytes = slots_n * n * 2 + slots_n * drafts * n * 2          # read 48 states + write 48 x 16 checkpoints
     kept = int((keep > 0).sum().item())
     sbytes = 2 * kept * n * 2
@@ -301,6 +326,8 @@ def bench_verify(steps, warmup, stream):
                      "frac": vbytes / (ms_v * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": TRAFFIC_BYTES["verify_chain"],
                      "kernel": "chain_kernel<bf16> with checkpoints", "bytes_per_launch": vbytes},
         "select_GBps": sbytes / (ms_s * 1e-3) / 1e9,
+        "saves_form": {"verify_ms_per_layer": ms_vs, "replay_commit_ms_per_layer": ms_r,
+                       "bytes_saved_per_layer": total * heads * 1284},
         "config": {"workload": "benchmark configuration 4: verify 48 slots x 16 drafts, bf16 state, per-row checkpoints; "
                                "select with keep ~ U{0..16}", "kept_slots": kept},
     }
