@@ -34,8 +34,8 @@ from glm53f_kda import DK, DV, HEADS, LAYERS, WINDOW, channels, ffi, state_len
 # offline; the summaries are kept in profiles/.
 TRAFFIC_BYTES = {
     "decode_chain": (36_805 + 33_024) * 1024,            # per chain launch, 16 slots x 1 row
-    "verify_chain": (226_538 + 1_585_152) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
-    "prefill_2048_rows": (135_598 + 148_845 + 152_700 + 36_864 + 65_571 + 32_768 + 172 + 144) * 1024,
+    "verify_chain": (167_932 + 1_585_152) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
+    "prefill_2048_rows": (141_315 + 148_482 + 152_700 + 36_864 + 65_571 + 32_768 + 172 + 144) * 1024,
 }
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
@@ -258,7 +258,7 @@ def bench_prefill(steps, warmup, stream, cpu=True):
 
 # ------------------------------------------------------------------------------------------------ verify
 
-def bench_verify(steps, warmup, stream):
+def bench_verify(steps, warmup, stream, saves_form=True):
     """benchmark configuration 4: 48 slots x 16 draft rows, bf16 state, a checkpoint after every row, then the commit by
     selection with an accepted length per slot drawn uniformly from [0, 16]."""
     heads, slots_n, drafts, layers = HEADS, 48, 16, 2
@@ -292,6 +292,21 @@ def bench_verify(steps, warmup, stream):
 
     ms_v = timed(verify, steps, warmup, stream)
     ms_s = timed(select, steps, warmup, stream)
+    vbytes = slots_n * n * 2 + slots_n * drafts * n * 2          # read 48 states + write 48 x 16 checkpoints
+    kept = int((keep > 0).sum().item())
+    sbytes = 2 * kept * n * 2
+
+    res = {
+        "verify_ms_per_layer": ms_v, "select_ms_per_layer": ms_s,
+        "roofline": {"bound": "hbm", "achieved": vbytes / (ms_v * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": vbytes / (ms_v * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": TRAFFIC_BYTES["verify_chain"],
+                     "kernel": "chain_kernel<bf16> with checkpoints", "bytes_per_launch": vbytes},
+        "select_GBps": sbytes / (ms_s * 1e-3) / 1e9,
+        "config": {"workload": "benchmark configuration 4: verify 48 slots x 16 drafts, bf16 state, per-row checkpoints; "
+                               "select with keep ~ U{0..16}", "kept_slots": kept},
+    }
+    if not saves_form:
+        return res
 
     # The reference's form of the same round, for comparison: the verify pass saves every row's replay inputs
     # (1,284 B per row and head) and leaves the state alone; the commit replays the kept prefix from the saves.
@@ -317,20 +332,9 @@ def bench_verify(steps, warmup, stream):
 
     ms_vs = timed(verify_saves, steps, warmup, stream)
     ms_r = timed(replay, steps, warmup, stream)
-    vbytes = slots_n * n * 2 + slots_n * drafts * n * 2          # read 48 states + write 48 x 16 checkpoints
-    kept = int((keep > 0).sum().item())
-    sbytes = 2 * kept * n * 2
-    return {
-        "verify_ms_per_layer": ms_v, "select_ms_per_layer": ms_s,
-        "roofline": {"bound": "hbm", "achieved": vbytes / (ms_v * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": vbytes / (ms_v * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": TRAFFIC_BYTES["verify_chain"],
-                     "kernel": "chain_kernel<bf16> with checkpoints", "bytes_per_launch": vbytes},
-        "select_GBps": sbytes / (ms_s * 1e-3) / 1e9,
-        "saves_form": {"verify_ms_per_layer": ms_vs, "replay_commit_ms_per_layer": ms_r,
-                       "bytes_saved_per_layer": total * heads * 1284},
-        "config": {"workload": "benchmark configuration 4: verify 48 slots x 16 drafts, bf16 state, per-row checkpoints; "
-                               "select with keep ~ U{0..16}", "kept_slots": kept},
-    }
+    res["saves_form"] = {"verify_ms_per_layer": ms_vs, "replay_commit_ms_per_layer": ms_r,
+                         "bytes_saved_per_layer": total * heads * 1284}
+    return res
 
 
 # ------------------------------------------------------------------------------------------------ main
@@ -385,7 +389,8 @@ def main():
                          "ms_per_step": pre["ms_per_8192_tokens"], "roofline": pre["roofline"],
                          "config": pre["config"]})
     if args.only in (None, "verify"):
-        ver = bench_verify(max(2, args.steps // 4), max(1, args.warmup // 2), stream)
+        # alone (--only verify) the leg runs the checkpoint form only, so that a profile of it holds one kind of launch
+        ver = bench_verify(max(2, args.steps // 4), max(1, args.warmup // 2), stream, saves_form=args.only is None)
         line["verify"] = ver
         if args.only == "verify":
             line.update({"value": ver["roofline"]["achieved"], "ms_per_step": ver["verify_ms_per_layer"],
