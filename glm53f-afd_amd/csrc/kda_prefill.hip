@@ -843,14 +843,51 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
 }
 
 // The gated RMSNorm over the bf16 read-outs the inter pass left in `out` (reference: kda_prefill.cu:542-570,
-// cpu.rs:361-376): a wave per (row, head), two values per lane.
+// cpu.rs:361-376). Sixteen lanes per (row, head), eight values per lane in 128-bit pieces when `wide` (rows of `out`
+// and the gate 16-byte aligned); else a wave per (row, head), two values per lane.
 __global__ void __launch_bounds__(THREADS) norm_kernel(int H, const int32_t* __restrict__ cu_rows, int rows1,
                                                        const bf16_t* __restrict__ G, long long g_stride,
                                                        const bf16_t* __restrict__ norm_w, float eps, bf16_t* out,
-                                                       long long out_stride) {
+                                                       long long out_stride, int wide) {
     const RowRange rr = request_rows(cu_rows, blockIdx.y, rows1);
     const long long tasks = (long long)rr.rows * H;
-    const int wpb = THREADS / 64, lane = threadIdx.x & 63;
+    const int lane = threadIdx.x & 63;
+    if (wide) {
+        const int sub = lane & 15;                                   // this lane's eight values: 8 sub .. 8 sub + 7
+        const u32x4 wv = *reinterpret_cast<const u32x4*>(norm_w + 8 * sub);
+        const int per_block = THREADS / 16;
+        for (long long task = (long long)blockIdx.x * per_block + (threadIdx.x >> 4); task < tasks;
+             task += (long long)gridDim.x * per_block) {
+            const long long r = rr.row0 + task / H;
+            const int h = (int)(task % H);
+            u32x4* o = reinterpret_cast<u32x4*>(out + r * out_stride + h * DV + 8 * sub);
+            const u32x4 yy = *o;
+            const u32x4 gg = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(G + r * g_stride + h * DV + 8 * sub));
+            float y[8], ss = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                y[2 * e] = __uint_as_float(yy[e] << 16);
+                y[2 * e + 1] = __uint_as_float(yy[e] & 0xffff0000u);
+                ss = __builtin_fmaf(y[2 * e], y[2 * e], ss);
+                ss = __builtin_fmaf(y[2 * e + 1], y[2 * e + 1], ss);
+            }
+            ss = ss + lane_xor16<1>(ss);
+            ss = ss + lane_xor16<2>(ss);
+            ss = ss + lane_xor16<4>(ss);
+            ss = ss + lane_xor16<8>(ss);
+            const float rinv = __builtin_amdgcn_rsqf(ss * (1.0f / (float)DV) + eps);
+            u32x4 res;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float g0 = __uint_as_float(gg[e] << 16), g1 = __uint_as_float(gg[e] & 0xffff0000u);
+                const float w0 = __uint_as_float(wv[e] << 16), w1 = __uint_as_float(wv[e] & 0xffff0000u);
+                res[e] = f2bf2(w0 * (y[2 * e] * rinv) * fast_sigmoid(g0), w1 * (y[2 * e + 1] * rinv) * fast_sigmoid(g1));
+            }
+            *o = res;
+        }
+        return;
+    }
+    const int wpb = THREADS / 64;
     const uint32_t wpair = reinterpret_cast<const uint32_t*>(norm_w)[lane];
     const float w0 = __uint_as_float(wpair << 16), w1 = __uint_as_float(wpair & 0xffff0000u);
     for (long long task = (long long)blockIdx.x * wpb + (threadIdx.x >> 6); task < tasks;
@@ -962,8 +999,9 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
         if (max_rows == 0) break;
     }
     if (max_rows > 0) {
+        const int wide = aligned16(out) && aligned16(g) && aligned16(norm_w) && out_stride % 8 == 0 && g_stride % 8 == 0;
         norm_kernel<<<dim3(kNormBlocks, batch), THREADS, 0, st>>>(heads, cu_rows, rows1, bfp(g), g_stride, bfp(norm_w),
-                                                                  eps, bfp(out), out_stride);
+                                                                  eps, bfp(out), out_stride, wide);
         const int rc = (int)hipGetLastError();
         if (rc != 0) return rc;
     }
