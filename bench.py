@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the KDA hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|mark|copy]
 
 Prints ONE JSON line. The headline `value` is the decode step's state traffic in GB/s in the 16-slot decode configuration
 (16 slots x 1 token out of a 48-slot bf16 pool, 64 heads, 34 layers each with its own pool so the working set
@@ -36,6 +36,7 @@ TRAFFIC_BYTES = {
     "decode_chain": (36_805 + 33_024) * 1024,            # per chain launch, 16 slots x 1 row
     "verify_chain": (167_932 + 1_585_152) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
     "prefill_2048_rows": (141_315 + 148_482 + 152_700 + 36_864 + 65_571 + 32_768 + 172 + 144) * 1024,
+    "mark_state_pages": (69_984 + 70_788) * 1024,
 }
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
@@ -337,6 +338,80 @@ def bench_verify(steps, warmup, stream, saves_form=True):
     return res
 
 
+# ------------------------------------------------------------------------------------------------ mark
+
+def bench_mark(steps, warmup, stream, cpu=True):
+    """A snapshot mark of one slot's positional state in the full model's layout with bf16 KDA states (195 pool
+    pages of 394,944 B; crates/glm53f-forward/src/kv.rs:412-478): the scatter of the state's 180 whole pages
+    alone, and the whole save and load as the engine runs them (page list upload, two launches, three copies of
+    partial pages)."""
+    from glm53f_forward import ffi as rf
+    from glm53f_forward.kv import KvPool
+    from glm53f_forward.kvplan import KvLayout
+    l = KvLayout().with_kda_state_bf16(True)
+    # Four slots and four marks in turn: 8 x 73 MiB, so that no call finds its source in the 256 MB Infinity Cache
+    # because the call before it left it there.
+    nslots = 4
+    pool = KvPool(l, slots=nslots, pages=2 * nslots * l.mark_pages() + 16)
+    gen = torch.Generator(device=DEV).manual_seed(6)
+    pool.state[:] = torch.randint(0, 256, (pool.state.numel(),), device=DEV, generator=gen, dtype=torch.uint8)
+    # every other page of the pool, so that a mark's pages are no contiguous run
+    held = [pool.alloc.alloc() for _ in range(2 * nslots * l.mark_pages())]
+    for pg in held[1::2]:
+        pool.alloc.release(pg)
+    kvs = [pool.slot() for _ in range(nslots)]
+    marks = [kv.mark() for kv in kvs]
+    torch.cuda.synchronize()
+    pb, full = l.page_bytes, l.kda_state_bytes() // l.page_bytes
+    lists = [torch.tensor(m.page_list(), dtype=torch.int32, device=DEV) for m in marks]
+    calls = [[ptr(pool.state, kv.state_at()), pb, ptr(ix), ptr(pool.pages), pb, full, pb, None]
+             for kv, ix in zip(kvs, lists)]
+    turn = [0]
+
+    def scatter():
+        turn[0] += 1
+        check(rf.glm53f_fwd_scatter_rows(*calls[turn[0] % nslots]), "scatter rows")
+
+    def save():
+        turn[0] += 1
+        kvs[turn[0] % nslots].copy_mark(marks[turn[0] % nslots], True)
+
+    def load():
+        turn[0] += 1
+        kvs[turn[0] % nslots].copy_mark(marks[turn[0] % nslots], False)
+
+    ms_scatter = timed(scatter, steps, warmup, stream)
+    ms_save = timed(save, steps, warmup, stream)
+    ms_load = timed(load, steps, warmup, stream)
+    m = marks[0]
+    moved = 2 * full * pb
+    res = {"config": {"workload": "snapshot mark of one slot, full model layout with bf16 KDA states: 195 pages "
+                                  "of 394,944 B (181 state, 13 conv, 1 tails), pages not contiguous; four slots and marks in turn",
+                      "mark_bytes": l.mark_bytes(), "pages": l.mark_pages()},
+           "scatter_state_pages_ms": ms_scatter, "save_ms": ms_save, "load_ms": ms_load,
+           "save_GBps": 2 * l.mark_bytes() / (ms_save * 1e-3) / 1e9,
+           "load_GBps": 2 * l.mark_bytes() / (ms_load * 1e-3) / 1e9,
+           "roofline": {"bound": "hbm", "kernel": "long_rows_kernel", "achieved": moved / (ms_scatter * 1e-3) / 1e9,
+                        "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                        "frac": moved / (ms_scatter * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                        "traffic": TRAFFIC_BYTES["mark_state_pages"],
+                        "algorithmic_bytes": moved}}
+    if cpu:
+        from oracle import rows_oracle as ro
+        image = np.random.default_rng(3).integers(0, 256, l.mark_bytes(), dtype=np.uint8)
+        s, c = l.kda_state_bytes(), l.conv_bytes()
+        arenas = [(image[:s], 0), (image[s:s + c], 0), (image[s + c:], 0)]
+        host_pages = np.zeros(pool.pages.numel(), dtype=np.uint8)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or time.perf_counter() - t0 < 2.0:
+            ro.copy_mark(l.mark_regions(), pb, m.page_list(), host_pages, arenas, True)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": 2 * l.mark_bytes() / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"{reps} saves of the same mark by the numpy restatement (page-sized memcpys)"}
+    return res
+
+
 # ------------------------------------------------------------------------------------------------ main
 
 # ------------------------------------------------------------------------------------------------ copy
@@ -356,7 +431,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", choices=["decode", "prefill", "verify", "copy"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "copy"], default=None)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -395,6 +470,12 @@ def main():
         if args.only == "verify":
             line.update({"value": ver["roofline"]["achieved"], "ms_per_step": ver["verify_ms_per_layer"],
                          "roofline": ver["roofline"], "config": ver["config"]})
+    if args.only in (None, "mark"):
+        mk = bench_mark(args.steps, args.warmup, stream, cpu=not args.no_cpu)
+        line["mark"] = mk
+        if args.only == "mark":
+            line.update({"value": mk["roofline"]["achieved"], "ms_per_step": mk["scatter_state_pages_ms"],
+                         "roofline": mk["roofline"], "config": mk["config"]})
     if args.only == "copy":
         cp = bench_copy(args.steps, args.warmup, stream)
         line.update({"copy": cp, "value": cp["GBps"], "ms_per_step": cp["ms"],
