@@ -5,8 +5,9 @@
 
 Prints ONE JSON line. The headline `value` is the decode step's state traffic in GB/s in the 16-slot decode configuration
 (16 slots x 1 token out of a 48-slot bf16 pool, 64 heads, 34 layers each with its own pool so the working set
-exceeds the last-level cache); a "step" is one decode step over the 34 KDA layers (chain + conv shift per
-layer). The same line carries the chunked prefill (T = 8192 as four sequential 2048-row calls on one
+exceeds the last-level cache); a "step" is one decode step over the 34 KDA layers: per layer the chain and the
+conv window advance, in one launch (the reference engine's two launches per layer are timed beside it as
+`decode_two_launches`). The same line carries the chunked prefill (T = 8192 as four sequential 2048-row calls on one
 slot) and the checkpointing verify (48 slots x 16 drafts) under `prefill` and `verify`, each with its
 own roofline object, and the CPU oracle timed on this host's cores as `cpu_baseline`.
 
@@ -96,8 +97,17 @@ class RowBuffers:
                       f(self.p[first:first + n, c:c + h]), f(self.g[first:first + n]))
 
 
+PREWARM_S = 0.1
+
+
 def timed(fn, steps, warmup, stream):
-    """W untimed calls, then exactly K timed ones between events on `stream`; returns ms per call."""
+    """W untimed calls, then exactly K timed ones between events on `stream`; returns ms per call. Before the W
+    calls the same work runs untimed for a tenth of a second: a leg that starts on an idle GPU otherwise measures
+    the clocks ramping up (the decode step read 5 % slower as the first leg than as a later one)."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < PREWARM_S:
+        fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -149,7 +159,13 @@ def bench_decode(steps, warmup, stream, cpu=True):
     def shift(l):
         check(shift_fn(*shift_args[l]), "conv_shift")
 
-    def step():
+    fused_fn = ffi.glm53f_kda_chain_shift_batch_bf16state
+
+    def step():                                          # a decode round as one launch per layer
+        for l in range(layers):
+            check(fused_fn(*chain_args[l]), "chain + shift")
+
+    def step_two_launches():                             # the reference engine's two launches per layer
         for l in range(layers):
             chain(l)
             shift(l)
@@ -159,11 +175,14 @@ def bench_decode(steps, warmup, stream, cpu=True):
             chain(l)
 
     ms_step = timed(step, steps, warmup, stream)
+    ms_two = timed(step_two_launches, steps, max(1, warmup // 2), stream)
     ms_chain = timed(chains_only, steps, max(1, warmup // 2), stream) / layers
     state_bytes = 2 * batch * n * 2                      # read + write of 16 bf16 states: 67,108,864 B
     res = {
         "ms_per_step": ms_step,
         "state_GBps": layers * state_bytes / (ms_step * 1e-3) / 1e9,
+        "two_launches": {"ms_per_step": ms_two, "state_GBps": layers * state_bytes / (ms_two * 1e-3) / 1e9,
+                         "what": "glm53f_kda_chain_batch_bf16state then glm53f_kda_conv_shift_batch per layer"},
         "roofline": {"bound": "hbm", "achieved": state_bytes / (ms_chain * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": state_bytes / (ms_chain * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": TRAFFIC_BYTES["decode_chain"],
@@ -452,8 +471,11 @@ def main():
         dec = bench_decode(args.steps, args.warmup, stream, cpu=not args.no_cpu)
         line.update({"value": dec["state_GBps"], "ms_per_step": dec["ms_per_step"], "roofline": dec["roofline"],
                      "config": {"workload": "configs[1]: decode, 16 slots x 1 token of a 48-slot bf16 pool, "
-                                            "H=64, dk=dv=128, 34 layers (one pool each), chain + conv shift per layer",
+                                            "H=64, dk=dv=128, 34 layers (one pool each), per layer the chain and "
+                                            "the conv window advance in one launch "
+                                            "(glm53f_kda_chain_shift_batch_bf16state)",
                                 "slots": 16, "pool_slots": 48, "heads": 64, "layers": 34}})
+        line["decode_two_launches"] = dec["two_launches"]
         if "cpu_baseline" in dec:
             line["cpu_baseline"] = dec["cpu_baseline"]
     if args.only in (None, "prefill"):

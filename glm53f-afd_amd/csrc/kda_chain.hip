@@ -45,12 +45,12 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1,
         const bf16_t* __restrict__ P, long long p_stride, long long b_off,
         const bf16_t* __restrict__ A, long long a_stride, const bf16_t* __restrict__ G, long long g_stride,
-        const bf16_t* __restrict__ conv, const long long* __restrict__ conv_off, const bf16_t* __restrict__ cw,
+        const bf16_t* conv, const long long* __restrict__ conv_off, const bf16_t* __restrict__ cw,
         const S* state_in, S* state_out, const long long* __restrict__ state_off,
         const float* __restrict__ a_log, const float* __restrict__ dt_bias, const bf16_t* __restrict__ norm_w,
         float eps, float lower, bf16_t* __restrict__ out, long long out_stride, S* __restrict__ ckpt,
         float* __restrict__ k_save, bf16_t* __restrict__ v_save, float* __restrict__ g_save,
-        float* __restrict__ b_save) {
+        float* __restrict__ b_save, int shift) {
     using M = StateMap<S>;
     constexpr int KPL = M::KPL;
     const long long C = 3LL * H * DK;
@@ -211,6 +211,28 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
     do {   // rows >= 1 here; a do-while leaves no zero-trip path that would keep the loaded state alive
         const long long gr = rr.row0 + r;
         prologue();
+        // shift: the request's conv window moves past all its rows, in place (what conv_shift_kernel does with
+        // keep = rows, reference kda.cu:258-277). The new window is taps 1..3 of the last row, staged in LDS as
+        // pieces 48..191; this workgroup is the only one that reads or writes its head's channels, and its last
+        // read of the window (this row's piece) landed before the prologue. Stored here, ahead of the update, the
+        // writes drain while the state is worked on.
+        if (shift && r + 1 == rows && t >= 48 && t < 192) {
+            const int j = t / 48, rem = t - 48 * j;
+            bf16_t* dst = const_cast<bf16_t*>(cs) + (long long)(j - 1) * C + (long long)(rem >> 4) * H * DK + h * DK +
+                          (rem & 15) * 8;
+            const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x_stage + t * 16);
+            if ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+                // nontemporal: lines left dirty in the L2 would be written back at the end of the kernel, on its
+                // critical path
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(dst));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    dst[2 * e] = (bf16_t)(v[e] & 0xffffu);
+                    dst[2 * e + 1] = (bf16_t)(v[e] >> 16);
+                }
+            }
+        }
         if constexpr (kPrefetch) {
             if (r + 1 < rows) {
                 xpiece = row_piece(r + 1);
@@ -409,7 +431,7 @@ int chain_batch_launch(int32_t heads, int32_t batch, const int32_t* cu_rows, con
                        S* state_out, const int64_t* state_off, const float* a_log, const float* dt_bias,
                        const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out, int64_t out_stride,
                        S* ckpt, float* k_save, glm53f_bf16* v_save, float* g_save, float* b_save,
-                       glm53f_stream_t stream) {
+                       glm53f_stream_t stream, int shift = 0) {
     if (batch < 1 || batch > 65535 || !cu_rows || !conv_off || !state_off ||
         !chain_args_ok(heads, p, a, g, conv, conv_w, state_in, a_log, dt_bias, norm_w, out, k_save, v_save, g_save,
                        b_save))
@@ -419,7 +441,7 @@ int chain_batch_launch(int32_t heads, int32_t batch, const int32_t* cu_rows, con
         heads, cu_rows, 0, bfp(p), p_stride, b_off, bfp(a), a_stride, bfp(g), g_stride, bfp(conv),
         reinterpret_cast<const long long*>(conv_off), bfp(conv_w), state_in, state_out,
         reinterpret_cast<const long long*>(state_off), a_log, dt_bias, bfp(norm_w), eps, lower, bfp(out), out_stride,
-        ckpt, k_save, bfp(v_save), g_save, b_save);
+        ckpt, k_save, bfp(v_save), g_save, b_save, shift);
     return launched();
 }
 
@@ -476,7 +498,7 @@ extern "C" int glm53f_kda_chain(int32_t heads, int32_t rows, const glm53f_bf16* 
     chain_kernel<float><<<dim3(heads, 1), THREADS, 0, (hipStream_t)stream>>>(
         heads, nullptr, rows, bfp(p), p_stride, b_off, bfp(a), a_stride, bfp(g), g_stride, bfp(conv), nullptr,
         bfp(conv_w), state_in, state_out, nullptr, a_log, dt_bias, bfp(norm_w), eps, lower, bfp(out), out_stride,
-        nullptr, k_save, bfp(v_save), g_save, b_save);
+        nullptr, k_save, bfp(v_save), g_save, b_save, 0);
     return launched();
 }
 
@@ -508,6 +530,37 @@ extern "C" int glm53f_kda_chain_batch_bf16state(int32_t heads, int32_t batch, co
                                       conv_off, conv_w, bfp(state_in), bfp(state_out), state_off, a_log, dt_bias,
                                       norm_w, eps, lower, out, out_stride, nullptr, k_save, v_save, g_save, b_save,
                                       stream);
+}
+
+extern "C" int glm53f_kda_chain_shift_batch(int32_t heads, int32_t batch, const int32_t* cu_rows, const glm53f_bf16* p,
+                                            int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride,
+                                            const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv,
+                                            const int64_t* conv_off, const glm53f_bf16* conv_w,
+                                            const float* state_in, float* state_out, const int64_t* state_off,
+                                            const float* a_log, const float* dt_bias, const glm53f_bf16* norm_w,
+                                            float eps, float lower, glm53f_bf16* out, int64_t out_stride,
+                                            float* k_save, glm53f_bf16* v_save, float* g_save, float* b_save,
+                                            glm53f_stream_t stream) {
+    return chain_batch_launch<float>(heads, batch, cu_rows, p, p_stride, b_off, a, a_stride, g, g_stride, conv,
+                                     conv_off, conv_w, state_in, state_out, state_off, a_log, dt_bias, norm_w, eps,
+                                     lower, out, out_stride, nullptr, k_save, v_save, g_save, b_save, stream, 1);
+}
+
+extern "C" int glm53f_kda_chain_shift_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,
+                                                      const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
+                                                      const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g,
+                                                      int64_t g_stride, glm53f_bf16* conv, const int64_t* conv_off,
+                                                      const glm53f_bf16* conv_w, const glm53f_bf16* state_in,
+                                                      glm53f_bf16* state_out, const int64_t* state_off,
+                                                      const float* a_log, const float* dt_bias,
+                                                      const glm53f_bf16* norm_w, float eps, float lower,
+                                                      glm53f_bf16* out, int64_t out_stride, float* k_save,
+                                                      glm53f_bf16* v_save, float* g_save, float* b_save,
+                                                      glm53f_stream_t stream) {
+    return chain_batch_launch<bf16_t>(heads, batch, cu_rows, p, p_stride, b_off, a, a_stride, g, g_stride, conv,
+                                      conv_off, conv_w, bfp(state_in), bfp(state_out), state_off, a_log, dt_bias,
+                                      norm_w, eps, lower, out, out_stride, nullptr, k_save, v_save, g_save, b_save,
+                                      stream, 1);
 }
 
 extern "C" int glm53f_kda_verify_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,

@@ -37,6 +37,10 @@ PROTOTYPES = {
     "glm53f_kda_verify_batch_bf16state": (C.c_int, [i32, i32, ptr] + _ROWS + [ptr, ptr, ptr, ptr, ptr] + _WEIGHTS
                                           + [ptr, i64, ptr] + _SAVES + [ptr]),
     "glm53f_kda_select_batch_bf16state": (C.c_int, [i32, i32, i32, ptr, ptr, ptr, i64, ptr, i64, ptr, ptr]),
+    "glm53f_kda_chain_shift_batch": (C.c_int, [i32, i32, ptr] + _ROWS + [ptr, ptr, ptr, ptr, ptr, ptr] + _WEIGHTS
+                                     + [ptr, i64] + _SAVES + [ptr]),
+    "glm53f_kda_chain_shift_batch_bf16state": (C.c_int, [i32, i32, ptr] + _ROWS + [ptr, ptr, ptr, ptr, ptr, ptr]
+                                               + _WEIGHTS + [ptr, i64] + _SAVES + [ptr]),
     "glm53f_kda_arch": (C.c_char_p, []),
 }
 

@@ -4,8 +4,9 @@
  * reference's crates/glm53f-kda/kernels/glm53f_kda.h:73-270, which its Rust bindings mirror in
  * crates/glm53f-kda/src/ffi.rs:16-287 and which crates/glm53f-forward calls directly
  * (src/forward.rs:1980-2039, :3585-3760). Only the stream handle changes: a HIP stream.
- * Three more entry points (end of this file) add the speculative-verify step with per-position state
- * checkpoints; they have no counterpart in the reference, whose rollback recomputes from saved rows.
+ * More entry points (end of this file) have no counterpart in the reference: the speculative-verify step
+ * with per-position state checkpoints (the reference's rollback recomputes from saved rows) and the decode
+ * round in one launch.
  *
  * Conventions (reference header :5-9): every pointer is a DEVICE pointer; strides and offsets count
  * ELEMENTS, not bytes; the return value is a hipError_t as int: 0 on success, 1 (hipErrorInvalidValue)
@@ -295,6 +296,40 @@ int glm53f_kda_select_batch_bf16state(int32_t heads, int32_t layers, int32_t bat
                                       const glm53f_bf16* ckpt, int64_t ckpt_layer_stride,
                                       glm53f_bf16* state, int64_t state_stride,
                                       const int64_t* state_off, glm53f_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * A decode round in one launch. No counterpart in the reference, whose engine runs the chain and then
+ * glm53f_kda_conv_shift_batch with keep = rows for every layer (crates/glm53f-forward/src/forward.rs:3669-3760);
+ * a single decode row's chain takes 15 us here and the shift's launch adds 4 us to it.
+ * ------------------------------------------------------------------------------------------------ */
+
+/**
+ * glm53f_kda_chain_batch followed by the advance of every request's conv window past all of its rows (the
+ * result of glm53f_kda_conv_shift_batch with keep[b] = rows of b, bit for bit), in the same launch. `conv` is
+ * written: the windows of different requests must not overlap. A request without rows keeps its window.
+ * Not for a verify round, whose windows must wait for the commit.
+ */
+int glm53f_kda_chain_shift_batch(int32_t heads, int32_t batch, const int32_t* cu_rows, const glm53f_bf16* p,
+                                 int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride,
+                                 const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv,
+                                 const int64_t* conv_off, const glm53f_bf16* conv_w, const float* state_in,
+                                 float* state_out, const int64_t* state_off, const float* a_log,
+                                 const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower,
+                                 glm53f_bf16* out, int64_t out_stride, float* k_save, glm53f_bf16* v_save,
+                                 float* g_save, float* b_save, glm53f_stream_t stream);
+
+/** glm53f_kda_chain_shift_batch with bf16 states in the pool (as glm53f_kda_chain_batch_bf16state). */
+int glm53f_kda_chain_shift_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,
+                                           const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
+                                           const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g,
+                                           int64_t g_stride, glm53f_bf16* conv, const int64_t* conv_off,
+                                           const glm53f_bf16* conv_w, const glm53f_bf16* state_in,
+                                           glm53f_bf16* state_out, const int64_t* state_off,
+                                           const float* a_log, const float* dt_bias,
+                                           const glm53f_bf16* norm_w, float eps, float lower,
+                                           glm53f_bf16* out, int64_t out_stride, float* k_save,
+                                           glm53f_bf16* v_save, float* g_save, float* b_save,
+                                           glm53f_stream_t stream);
 
 /** The gfx architecture the kernels were compiled for ("gfx950"). */
 const char* glm53f_kda_arch(void);

@@ -204,9 +204,10 @@ class Pool:
 
 
 def chain_batch_gpu(p: o.LayerParams, pool: Pool, slots: list[int], reqs: list[o.Rows], *, write="inplace",
-                    saves=False, ckpt=False, pad=0):
+                    saves=False, ckpt=False, pad=0, shift=False):
     """glm53f_kda_chain_batch[_bf16state] / verify over requests living in `slots` of `pool`.
-    write: "inplace", "skip" or "to" (a fresh buffer). Returns (out rows, state tensor or None, Saves, ckpt)."""
+    write: "inplace", "skip" or "to" (a fresh buffer). shift: the entry points that also advance the conv windows
+    of the pool. Returns (out rows, state tensor or None, Saves, ckpt)."""
     w = Weights(p)
     sr = StagedRows(stack_rows(reqs), pad=pad)
     meta = BatchMeta([r.rows for r in reqs], [pool.conv_off(s) for s in slots], [pool.state_off(s) for s in slots])
@@ -227,7 +228,10 @@ def chain_batch_gpu(p: o.LayerParams, pool: Pool, slots: list[int], reqs: list[o
         code = ffi.glm53f_kda_verify_batch_bf16state(*common, ptr(meta.state_off), *tail, ptr(ck),
                                                      *(sv.args() if sv else NO_SAVES), None)
     else:
-        fn = ffi.glm53f_kda_chain_batch_bf16state if pool.bf16 else ffi.glm53f_kda_chain_batch
+        if shift:
+            fn = ffi.glm53f_kda_chain_shift_batch_bf16state if pool.bf16 else ffi.glm53f_kda_chain_shift_batch
+        else:
+            fn = ffi.glm53f_kda_chain_batch_bf16state if pool.bf16 else ffi.glm53f_kda_chain_batch
         code = fn(*common, ptr(s_out), ptr(meta.state_off), *tail, *(sv.args() if sv else NO_SAVES), None)
     check(code, "chain_batch")
     sync()

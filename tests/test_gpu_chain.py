@@ -411,3 +411,57 @@ def test_conv_shift_wide_and_narrow_paths_agree_with_the_oracle():
     hs.check(ffi.glm53f_kda_conv_shift(cc, 2, hs.ptr(win), hs.ptr(p), cc, None), "conv shift")
     hs.sync()
     assert torch.equal(win.view(3, cc), torch.cat([before.view(3, cc)[2:], p.view(2, cc)]))
+
+
+@pytest.mark.parametrize("bf16_state", [False, True], ids=["f32-state", "bf16-state"])
+def test_chain_with_the_window_advance_in_one_launch(bf16_state):
+    """glm53f_kda_chain_shift_batch[_bf16state] == the chain, then glm53f_kda_conv_shift_batch with keep = rows
+    (what a decode round of the engine runs per layer), bit for bit: outputs, states, saves and windows; requests of
+    0, 1, 2, 3 and 7 rows in shuffled slots; a slot outside the batch is untouched."""
+    heads, slots = 6, [4, 1, 5, 0, 2]
+    p = o.synth_layer(heads, 61)
+    reqs = [o.synth_rows(heads, n, 70 + n) for n in (1, 0, 3, 7, 2)]
+    c = channels(heads)
+    two = hs.Pool(heads, 6, bf16_state, 62)
+    one = hs.Pool(heads, 6, bf16_state, 62)
+    out2, st2, sv2, _, m2 = hs.chain_batch_gpu(p, two, slots, reqs, saves=True)
+    sr = hs.StagedRows(hs.stack_rows(reqs))
+    hs.check(ffi.glm53f_kda_conv_shift_batch(c, 1, m2.batch, hs.ptr(m2.cu_rows), hs.ptr(m2.keep), hs.ptr(two.conv), 0,
+                                             hs.ptr(m2.conv_off), hs.ptr(sr.p), 0, sr.p_stride, None), "conv shift")
+    hs.sync()
+    out1, st1, sv1, _, _ = hs.chain_batch_gpu(p, one, slots, reqs, saves=True, shift=True)
+    assert np.array_equal(hs.bits(out1), hs.bits(out2))
+    assert torch.equal(st1, st2)
+    for a, b in zip((sv1.k, sv1.v, sv1.g, sv1.b), (sv2.k, sv2.v, sv2.g, sv2.b)):
+        assert torch.equal(a, b)
+    assert torch.equal(one.conv, two.conv)
+    for i, slot in enumerate(slots):
+        want = o.conv_shift(one.conv_of(slot), reqs[i], reqs[i].rows)
+        at = one.conv_off(slot)
+        assert np.array_equal(hs.back(one.conv[at:at + WINDOW * c]), want), slot
+    at = one.conv_off(3)
+    assert np.array_equal(hs.back(one.conv[at:at + WINDOW * c]), one.conv_of(3))
+
+
+def test_chain_with_the_window_advance_on_unaligned_windows():
+    """A window that starts 2 bytes off a 16-byte boundary is read and written in 16-bit elements."""
+    heads = 2
+    p = o.synth_layer(heads, 63)
+    rows = o.synth_rows(heads, 2, 64)
+    c = channels(heads)
+    w = hs.Weights(p)
+    sr = hs.StagedRows(rows)
+    pool = hs.Pool(heads, 1, True, 65)
+    conv_host = pool.conv_of(0)
+    shifted = torch.zeros(WINDOW * c + 8, dtype=torch.bfloat16, device=hs.DEV)
+    shifted[1:1 + WINDOW * c] = pool.conv
+    meta = hs.BatchMeta([2], [0], [0])
+    hs.check(ffi.glm53f_kda_chain_shift_batch_bf16state(
+        heads, 1, hs.ptr(meta.cu_rows), *sr.row_args(), hs.ptr(shifted, 1), hs.ptr(meta.conv_off), hs.ptr(w.conv_w),
+        hs.ptr(pool.state), hs.ptr(pool.state), hs.ptr(meta.state_off), *w.args(), hs.ptr(sr.out), sr.out_stride,
+        *hs.NO_SAVES, None), "chain + shift")
+    hs.sync()
+    assert np.array_equal(hs.back(shifted[1:1 + WINDOW * c]), o.conv_shift(conv_host, rows, 2))
+    assert float(shifted[0]) == 0.0 and float(shifted[1 + WINDOW * c]) == 0.0
+    ref = o.chain_bf16_state(p, conv_host, pool.state_of(0), rows)
+    assert hs.rel_err(pool.device_state(0), ref.state) <= 1e-2
