@@ -69,431 +69,340 @@ __device__ __forceinline__ f32x4 mfma_f16(uint4 a, uint4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
-// C[16][16] += A[a_row0 ..][0, K) . B^T[b_row0 ..][0, K) with fp16 operands.
-__device__ __forceinline__ f32x4 tile_f16(const uint16_t* a, int a_row0, int lda, const uint16_t* b, int b_row0, int ldb,
-                                          int K, int lane, f32x4 acc) {
-    for (int k0 = 0; k0 < K; k0 += 32) acc = mfma_f16(frag(a, lda, a_row0, k0, lane), frag(b, ldb, b_row0, k0, lane), acc);
-    return acc;
-}
-
-// C[16][16] += A[a_row0 ..][0, 128) . B^T[b_row0 ..][0, 128) with f32 operands (v_mfma_f32_16x16x4_f32: lanes
-// 16 g .. 16 g + 15 supply one k per instruction). Which k a lane group supplies at which step is free as long as
-// both operands agree, so group g walks k = 32 g .. 32 g + 31 and reads its 32 values as eight 128-bit pieces.
-constexpr int LDG = DK + 4;                       // f32 row stride of these operands
-__device__ __forceinline__ f32x4 tile_f32(const float* a, int a_row0, const float* b, int b_row0, int lane, f32x4 acc) {
-    const f32x4* pa = reinterpret_cast<const f32x4*>(a + (a_row0 + (lane & 15)) * LDG + 32 * (lane >> 4));
-    const f32x4* pb = reinterpret_cast<const f32x4*>(b + (b_row0 + (lane & 15)) * LDG + 32 * (lane >> 4));
-#pragma unroll
-    for (int p = 0; p < 8; ++p) {
-        const f32x4 va = pa[p], vb = pb[p];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(va[e], vb[e], acc, 0, 0, 0);
-    }
-    return acc;
-}
-
-// LDS map of intra_kernel, bytes.
-constexpr int I_TOT = 0;                          // f32 [4][128]: log-decay totals of the sub-chunks
+// LDS map of intra_kernel, bytes. 75.5 KB: two workgroups share a CU.
+constexpr int LDD = SUB + 4;                      // f32 row stride of a diagonal block of L (16-byte multiple)
+constexpr int LDT = 40, LDZ = 24;                 // 16-bit row strides of TT and Z (16-byte multiples)
+constexpr int NFAC = 14;                          // per-channel factors between sub-chunks (see factor_index)
+constexpr int I_CW = 0;                           // bf16 [q | k | v][128 channels][4 taps]: the head's conv weights
+constexpr int I_DTB = I_CW + 3 * DK * TAPS * 2;   // f32 [128]: the head's dt_bias
+constexpr int I_TOT = I_DTB + DK * 4;             // f32 [4][128]: log-decay totals of the sub-chunks
 constexpr int I_BETA = I_TOT + 4 * DK * 4;        // f32 [64]
-constexpr int I_INV = I_BETA + CH * 4;            // f32 [2][64]: 1/|q| * 128^-0.5, 1/|k|
-constexpr int I_KET = I_INV + 2 * CH * 4;         // fp16 [128 keys][LD64]: k e^G, transposed
+constexpr int I_KET = I_BETA + CH * 4;            // fp16 [128 keys][LD64]: k e^G, transposed
 constexpr int I_VT = I_KET + DK * LD64 * 2;       // fp16 [128 values][LD64]: v, transposed
 constexpr int I_LN = I_VT + DV * LD64 * 2;        // fp16 [64][LD64]: -L below the block diagonal, zero elsewhere
-constexpr int LDD = SUB + 4;                      // f32 row stride of a diagonal block of L (16-byte multiple)
 constexpr int I_LD = I_LN + CH * LD64 * 2;        // f32 [4][16][LDD]: the diagonal blocks of L
-constexpr int I_KC1 = I_LD + 4 * SUB * LDD * 4;   // fp16 [32][LD128]: column side around the chunk's middle
-constexpr int I_PASS = I_KC1 + 32 * LD128 * 2;    // the rest is reused by every half
-constexpr int P_ROWS32 = 32 * LD128 * 2;          // one [32][LD128] 16-bit array
-constexpr int P_ROWS16 = 16 * LD128 * 2;
-constexpr int I_DIAG = I_PASS;                    // three f32 [32][LDG] arrays: KrD, QrD, KcD (within six P_ROWS32)
-constexpr int I_RAWQ = I_PASS;                    // raw q, k (bf16) before the norms: dead before the operands land
-constexpr int I_RAWK = I_PASS + P_ROWS32;
-constexpr int I_R2 = I_DIAG + 6 * P_ROWS32;       // KR2, QR2, KC2: three [16][LD128] fp16 arrays
-constexpr int I_R1 = I_R2 + 3 * P_ROWS16;         // KR1, QR1: two [32][LD128] fp16 arrays
-constexpr int I_END = I_R1 + 2 * P_ROWS32;
-// After the halves: the block solve.
-constexpr int LDT = 40, LDZ = 24;                 // 16-bit row strides of the two arrays below (16-byte multiples)
-constexpr int I_TT = I_PASS;                      // fp16 [64][LDT]: row 16 a + i holds [T_aa diag(beta) | T_aa][i][0..32)
-constexpr int I_Z = I_TT + CH * LDT * 2;          // fp16 [16 column tiles][16][LDZ]: a tile of Z on its way back in
-// Input staging (before the operands of a half land): the half's 35 rows of q | k | v, and the chunk's gate rows.
-constexpr int LDX = DK + 8;                       // staged input rows, 16-bit elements
-constexpr int XROWS = 32 + WINDOW;
-constexpr int I_XIN = I_R2;                       // bf16 [3][35][LDX]
-constexpr int I_AIN = I_PASS;                     // bf16 [64][LDX]
-static_assert(I_XIN + 3 * XROWS * LDX * 2 <= I_END, "input staging must fit behind the diagonal operands");
-static_assert(3 * 32 * LDG * 4 <= 6 * P_ROWS32, "the f32 diagonal operands fit their region");
-constexpr int INTRA_LDS = I_END;
-constexpr int INTRA_CPW = 4;                     // consecutive chunks of a head per intra workgroup
-static_assert(I_Z + 16 * SUB * LDZ * 2 <= I_END, "solve scratch must fit the per-half region");
-static_assert(INTRA_LDS <= 160 * 1024, "intra_kernel LDS");
+constexpr int I_KCE = I_LD + 4 * SUB * LDD * 4;   // fp16 [3][16][LD128]: k e^{G_end - G} of sub-chunks 0..2, row major
+constexpr int I_Z = I_KCE;                        //   later fp16 [16 column tiles][16][LDZ]: a tile of Z on its way back
+constexpr int I_FAC = I_KCE + 3 * SUB * LD128 * 2;  // f32 [NFAC][128]
+constexpr int I_TT = I_FAC;                       //   later fp16 [64][LDT]: row 16 a + i holds [T_aa diag(beta) | T_aa][i][0..32)
+constexpr int INTRA_LDS = I_FAC + NFAC * DK * 4;
+constexpr int INTRA_CPW = 4;                      // consecutive chunks of a head per intra workgroup
+static_assert(16 * SUB * LDZ * 2 <= 3 * SUB * LD128 * 2, "Z fits the region of the column operands");
+static_assert(CH * LDT * 2 <= NFAC * DK * 4, "TT fits the region of the factors");
+static_assert(2 * INTRA_LDS <= 160 * 1024, "two intra workgroups per CU");
 
-// NROWS rows of 128 bf16 on their way from global memory to LDS rows of LDX elements. src(row) is the row's
-// address or nullptr for a row of zeros. With `vec` every row is 16-byte aligned and moves in 128-bit pieces:
-// load() issues all of a lane's loads at once, store() lands them later, so the memory latency hides behind
-// whatever runs in between. Without `vec` store() copies 16-bit elements directly.
-template <int NROWS>
-struct StagedRows {
-    static constexpr int PIECES = NROWS * 16, IT = (PIECES + THREADS - 1) / THREADS;
-    u32x4 x[IT];
-    template <typename F>
-    __device__ __forceinline__ void load(F src, bool vec, int t) {
-        if (!vec) return;
-#pragma unroll
-        for (int q = 0; q < IT; ++q) {
-            const int v = q * THREADS + t, row = v >> 4;
-            const bf16_t* p = v < PIECES ? src(row) : nullptr;
-            // nontemporal: the rows are read once, and plain loads would push the workspace this kernel writes for
-            // the next one out of the caches (measured: the next kernel runs 15 % faster)
-            x[q] = p != nullptr ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (v & 15) * 8))
-                                : u32x4{0u, 0u, 0u, 0u};
-        }
-    }
-    template <typename F>
-    __device__ __forceinline__ void store(uint16_t* dst, F src, bool vec, int t) const {
-        if (vec) {
-#pragma unroll
-            for (int q = 0; q < IT; ++q) {
-                const int v = q * THREADS + t;
-                if (v < PIECES) *reinterpret_cast<u32x4*>(dst + (v >> 4) * LDX + (v & 15) * 8) = x[q];
-            }
-        } else {
-            constexpr int ELEMS = NROWS * DK, ITE = (ELEMS + THREADS - 1) / THREADS;
-#pragma unroll 8
-            for (int q = 0; q < ITE; ++q) {
-                const int e = q * THREADS + t, row = e >> 7;
-                if (e < ELEMS) {
-                    const bf16_t* p = src(row);
-                    dst[row * LDX + (e & 127)] = p != nullptr ? p[e & 127] : (bf16_t)0;
-                }
-            }
-        }
-    }
-};
+// Factors e^{sum of whole sub-chunks' log decay}, per key channel: 0..3 = e^{G before sub-chunk a};
+// 4..7 = e^{G_last - G at the end of sub-chunk a}; 8 + a (a - 1) / 2 + b = e^{G at the start of a - G at the end of b}
+// for b < a (1 when they are neighbours).
+__device__ __forceinline__ int factor_index(int a, int b) { return 8 + a * (a - 1) / 2 + b; }
 
-// Pass 1: one chunk of one head of one request, everything that does not need the state, into its workspace slot.
-__global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) intra_kernel(
+// DPP moves inside a row of 16 lanes: the value n lanes below (0 where there is none), and lane n's value.
+template <int N>
+__device__ __forceinline__ float row_shr(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x110 + N, 0xf, 0xf, false));
+}
+template <int N>
+__device__ __forceinline__ float row_lane(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x150 + N, 0xf, 0xf, false));
+}
+
+// Eight consecutive bf16 from p. With VEC p is 16-byte aligned.
+template <bool VEC>
+__device__ __forceinline__ u32x4 load8(const bf16_t* p) {
+    if constexpr (VEC) {
+        return *reinterpret_cast<const u32x4*>(p);
+    } else {
+        u32x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (uint32_t)p[2 * e] | ((uint32_t)p[2 * e + 1] << 16);
+        return v;
+    }
+}
+__device__ __forceinline__ float bf_at(const u32x4 v, int e) {   // element e of eight packed bf16
+    return (e & 1) ? __uint_as_float(v[e >> 1] & 0xffff0000u) : __uint_as_float(v[e >> 1] << 16);
+}
+__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) { return (uint32_t)f2h(lo) | ((uint32_t)f2h(hi) << 16); }
+
+// Pass 1: the chunks of one head of one request, everything that does not need the state, into their workspace
+// slots. Wave w owns sub-chunk w of a chunk (rows 16 w .. 16 w + 15); in the elementwise phases lane l holds row
+// l % 16 and the 32 channels 32 (l / 16) .. + 31 of it. That is the operand layout of the matrix cores for
+// products that contract over channels, so the tiles of L and M take their row side straight from registers (the
+// diagonal ones both sides); what contracts over rows later (k e^G, v, Kg) is written transposed, 16 bits at a time.
+template <bool VEC>
+__global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) intra_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
         const bf16_t* __restrict__ P, long long p_stride, long long b_off, const bf16_t* __restrict__ A,
         long long a_stride, const bf16_t* __restrict__ conv, const long long* __restrict__ conv_off,
         const bf16_t* __restrict__ cw, const float* __restrict__ a_log, const float* __restrict__ dt_bias, float lower,
-        int vec, unsigned char* __restrict__ ws) {
+        unsigned char* __restrict__ ws) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int c_first = blockIdx.x * INTRA_CPW, h = blockIdx.y, b = blockIdx.z;
     const RowRange rr = request_rows(cu_rows, b, rows1);
     if (rr.rows - (sub0 + c_first * CH) <= 0) return;
-    // t, and what derives from it, are re-made at the top of every chunk from a value the optimizer cannot see
-    // through: otherwise the hundreds of per-lane addresses of the body are hoisted out of the chunk loop and
-    // spill.
-    int t = threadIdx.x, wave = t >> 6, lane = t & 63;
-    int d = t & (DK - 1), s = t >> 7;             // this lane's channel, and which sub-chunk of a half it takes
+    int t = threadIdx.x;
     const long long C = 3LL * H * DK;
     const bf16_t* cs = conv + (conv_off != nullptr ? conv_off[b] : 0);
 
+    uint2* cw_s = reinterpret_cast<uint2*>(smem + I_CW);            // [3 * 128] channels, four taps each
+    float* dtb_s = reinterpret_cast<float*>(smem + I_DTB);
     float* tot = reinterpret_cast<float*>(smem + I_TOT);
     float* beta_s = reinterpret_cast<float*>(smem + I_BETA);
-    float* inv_s = reinterpret_cast<float*>(smem + I_INV);
     uint16_t* keT = reinterpret_cast<uint16_t*>(smem + I_KET);
     uint16_t* VT = reinterpret_cast<uint16_t*>(smem + I_VT);
     uint16_t* Ln = reinterpret_cast<uint16_t*>(smem + I_LN);
     float* Ld = reinterpret_cast<float*>(smem + I_LD);
-    uint16_t* KC1 = reinterpret_cast<uint16_t*>(smem + I_KC1);
+    uint16_t* KcE = reinterpret_cast<uint16_t*>(smem + I_KCE);
+    float* fac = reinterpret_cast<float*>(smem + I_FAC);
 
-    // ---- gates of the whole chunk: cumulative log decay of this lane's channel inside its two sub-chunks
-    // Row `rel` (relative to the request's first row; -3..-1 are the conv window) of q | k | v, nullptr past the end.
-    auto input_row = [&](int rel) -> const bf16_t* {
-        if (rel >= rr.rows) return nullptr;
-        return rel < 0 ? cs + (long long)(rel + WINDOW) * C : P + (rr.row0 + rel) * p_stride;
-    };
-    // segment seg (q, k, v) of the input rows of half h2 of the chunk starting at row first, three rows before
-    // the half's first included
-    auto x_src = [&](int first, int h2, int seg) {
-        return [=](int j) -> const bf16_t* {
-            const bf16_t* row = input_row(first + 32 * h2 - WINDOW + j);
-            return row != nullptr ? row + seg * H * DK + h * DK : nullptr;
-        };
-    };
-    auto a_src = [&](int first) {
-        return [=](int R) -> const bf16_t* {
-            return first + R < rr.rows ? A + (rr.row0 + first + R) * a_stride + h * DK : nullptr;
-        };
-    };
-    // A workgroup takes INTRA_CPW consecutive chunks of its head. Every global input of a chunk's first half is
-    // requested while the chunk before it is still being worked on (for the first chunk: now); the second half's
-    // follows while the first half computes.
-    StagedRows<CH> a_st;
-    StagedRows<XROWS> x_st[3];
-    a_st.load(a_src(sub0 + c_first * CH), vec != 0, t);
-#pragma unroll
-    for (int seg = 0; seg < 3; ++seg) x_st[seg].load(x_src(sub0 + c_first * CH, 0, seg), vec != 0, t);
-    // the beta logit of row t of the chunk (lanes 0..63), requested with the rest of the chunk's inputs
-    auto beta_logit = [&](int first) -> bf16_t {
-        const int R = first + (t & (CH - 1));
-        return R < rr.rows ? P[(rr.row0 + R) * p_stride + b_off + h] : (bf16_t)0;
-    };
-    bf16_t b_raw = beta_logit(sub0 + c_first * CH);
+    // the head's conv weights and dt_bias, once (the first barrier of the chunk loop publishes them... they are
+    // read before it, so one barrier here)
+    for (int e = t; e < 3 * DK; e += THREADS)
+        cw_s[e] = *reinterpret_cast<const uint2*>(cw + ((size_t)(e >> 7) * H * DK + (size_t)h * DK + (e & (DK - 1))) * TAPS);
+    if (t < DK) dtb_s[t] = dt_bias[h * DK + t];
     const float rate = fast_exp(a_log[h]);
-    const float dtb = dt_bias[h * DK + d];
-    // conv weights of this lane's q, k and v channels
-    const unsigned cq = (unsigned)(h * DK + d), ck = (unsigned)(H * DK + h * DK + d), cv = (unsigned)(2 * H * DK + h * DK + d);
-    float wq[TAPS], wk[TAPS], wv[TAPS];
-    {
-        const uint2 a4 = *reinterpret_cast<const uint2*>(cw + (size_t)cq * TAPS);
-        const uint2 b4 = *reinterpret_cast<const uint2*>(cw + (size_t)ck * TAPS);
-        const uint2 c4 = *reinterpret_cast<const uint2*>(cw + (size_t)cv * TAPS);
-        wq[0] = __uint_as_float(a4.x << 16); wq[1] = __uint_as_float(a4.x & 0xffff0000u);
-        wq[2] = __uint_as_float(a4.y << 16); wq[3] = __uint_as_float(a4.y & 0xffff0000u);
-        wk[0] = __uint_as_float(b4.x << 16); wk[1] = __uint_as_float(b4.x & 0xffff0000u);
-        wk[2] = __uint_as_float(b4.y << 16); wk[3] = __uint_as_float(b4.y & 0xffff0000u);
-        wv[0] = __uint_as_float(c4.x << 16); wv[1] = __uint_as_float(c4.x & 0xffff0000u);
-        wv[2] = __uint_as_float(c4.y << 16); wv[3] = __uint_as_float(c4.y & 0xffff0000u);
-    }
+    __syncthreads();
+
 #pragma unroll 1
     for (int c = c_first; c < min(chunks, c_first + INTRA_CPW); ++c) {
+    // t, and what derives from it, are re-made for every chunk from a value the optimizer cannot see through:
+    // otherwise the per-lane addresses of the body are hoisted out of the chunk loop and spill.
     asm volatile("" : "+v"(t));
-    wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    lane = t & 63;
-    d = t & (DK - 1);
-    s = __builtin_amdgcn_readfirstlane(t >> 7);   // uniform inside a wave
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63;
+    const int i = lane & 15, g = lane >> 4;       // this lane's row of the sub-chunk and its group of 32 channels
     const int r0 = sub0 + c * CH;                 // the chunk's first row inside the request
     const int n = min(CH, rr.rows - r0);          // its real rows
     if (n <= 0) break;
-    const bool more = c + 1 < min(chunks, c_first + INTRA_CPW) && rr.rows - (r0 + CH) > 0;
+    const int R = SUB * wave + i;                 // this lane's row inside the chunk
     unsigned char* wsc = ws + (((long long)b * H + h) * chunks + c) * (long long)WS_BYTES;
-    uint16_t* ain = reinterpret_cast<uint16_t*>(smem + I_AIN);
-    a_st.store(ain, a_src(r0), vec != 0, t);
-    __syncthreads();
-    float cg[2][SUB];                             // inclusive cumulative sums, sub-chunks s and 2 + s
-#pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2) {
-        const int a = 2 * h2 + s;
-        float run = 0.0f;
-#pragma unroll
-        for (int i = 0; i < SUB; ++i) {
-            // rows past the end have g = 0; evaluated for every row and masked (a branch here would serialize
-            // the sixteen LDS reads and transcendentals)
-            const int R = SUB * a + i;
-            const float gv = lower * fast_sigmoid(rate * (bf2f(ain[R * LDX + d]) + dtb));
-            run += __uint_as_float(__float_as_uint(gv) & (R < n ? 0xffffffffu : 0u));
-            cg[h2][i] = run;
-        }
-        tot[a * DK + d] = run;
-    }
-    if (t < CH) beta_s[t] = t < n ? bfround(fast_sigmoid(bf2f(b_raw))) : 0.0f;
-    __syncthreads();
-    // prefix and suffix totals of this lane's channel: B[a] = sum of tot over sub-chunks before a
-    float Bp[5];
-    Bp[0] = 0.0f;
-#pragma unroll
-    for (int a = 0; a < 4; ++a) Bp[a + 1] = Bp[a] + tot[a * DK + d];
-    if (s == 0) reinterpret_cast<float*>(wsc + WS_E)[d] = fast_exp(Bp[4]);
 
-    // ---- the two halves of the chunk: sub-chunks {0, 1}, then {2, 3} (unrolled: h2 indexes registers)
+    // ---- conv + SiLU with one bf16 rounding (q, k stay in registers; v goes to VT as fp16, exact but for values
+    // below 2^-14), and the sums of squares for the L2 norms. Rows past the request's end are not masked: their
+    // beta is zero, which removes them from L, W, U and the state update, and their outputs are never stored.
+    uint32_t qr[16], kr[16];                      // bf16 pairs: the conv outputs are bf16 values
+    float ssq = 0.0f, ssk = 0.0f;
+    {
+        // a tap row past the end only feeds rows past the end: it reads the last real row instead
+        const bf16_t* rowp[TAPS];
 #pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2) {
-        const int a = 2 * h2 + s;                 // this lane's sub-chunk
-        const int lr0 = SUB * s;                  // its first row inside the half's 32-row arrays
-        uint16_t* rawq = reinterpret_cast<uint16_t*>(smem + I_RAWQ);
-        uint16_t* rawk = reinterpret_cast<uint16_t*>(smem + I_RAWK);
-        // the half's input rows (three before its first row included) into LDS, q | k | v side by side
-        uint16_t* xin = reinterpret_cast<uint16_t*>(smem + I_XIN);
-#pragma unroll
-        for (int seg = 0; seg < 3; ++seg) x_st[seg].store(xin + seg * XROWS * LDX, x_src(r0, h2, seg), vec != 0, t);
-        __syncthreads();
-        if (h2 == 0) {
-#pragma unroll
-            for (int seg = 0; seg < 3; ++seg) x_st[seg].load(x_src(r0, 1, seg), vec != 0, t);
-        } else if (more) {
-            b_raw = beta_logit(r0 + CH);
-            a_st.load(a_src(r0 + CH), vec != 0, t);
-#pragma unroll
-            for (int seg = 0; seg < 3; ++seg) x_st[seg].load(x_src(r0 + CH, 0, seg), vec != 0, t);
+        for (int tap = 0; tap < TAPS; ++tap) {
+            const int rel = min(r0 + R - WINDOW + tap, rr.rows - 1);
+            rowp[tap] = (rel < 0 ? cs + (long long)(rel + WINDOW) * C : P + (rr.row0 + rel) * p_stride) + h * DK + 32 * g;
         }
-        // conv + SiLU, one bf16 rounding, 16 rows of q, k, v
-        float qr[SUB], kr[SUB];
-        {
-            const uint16_t* xq_l = xin + (SUB * s) * LDX + d;                 // row j of the lane's sub-chunk: + j * LDX
-            const uint16_t* xk_l = xq_l + XROWS * LDX;
-            const uint16_t* xv_l = xk_l + XROWS * LDX;
-            // all 19 input rows of the three channels into registers first: the stores below go to the same
-            // memory, and reads issued between them would each wait out a full LDS latency
-            float xq[SUB + WINDOW], xk[SUB + WINDOW], xv[SUB + WINDOW];
+        u32x4 x[TAPS], xn[TAPS];
 #pragma unroll
-            for (int j = 0; j < SUB + WINDOW; ++j) {
-                xq[j] = bf2f(xq_l[j * LDX]);
-                xk[j] = bf2f(xk_l[j * LDX]);
-                xv[j] = bf2f(xv_l[j * LDX]);
+        for (int tap = 0; tap < TAPS; ++tap) x[tap] = load8<VEC>(rowp[tap]);
+#pragma unroll
+        for (int it = 0; it < 12; ++it) {
+            const int seg = it >> 2, p = it & 3;
+            if (it + 1 < 12) {
+                const int seg1 = (it + 1) >> 2, p1 = (it + 1) & 3;
+#pragma unroll
+                for (int tap = 0; tap < TAPS; ++tap)
+                    xn[tap] = load8<VEC>(rowp[tap] + (long long)seg1 * H * DK + 8 * p1);
             }
-            uint32_t vpack[SUB / 2];
 #pragma unroll
-            for (int i = 0; i < SUB; ++i) {
-                float aq = 0.0f, ak = 0.0f, av = 0.0f;
+            for (int e2 = 0; e2 < 4; ++e2) {      // two channels per 128-bit piece of weights
+                const u32x4 w2 = *reinterpret_cast<const u32x4*>(cw_s + seg * DK + 32 * g + 8 * p + 2 * e2);
+                float s2[2];
 #pragma unroll
-                for (int tap = 0; tap < TAPS; ++tap) {
-                    aq = __builtin_fmaf(wq[tap], xq[i + tap], aq);
-                    ak = __builtin_fmaf(wk[tap], xk[i + tap], ak);
-                    av = __builtin_fmaf(wv[tap], xv[i + tap], av);
+                for (int k = 0; k < 2; ++k) {
+                    const int e = 2 * e2 + k;
+                    const uint32_t wa = w2[2 * k], wb = w2[2 * k + 1];
+                    float acc = 0.0f;
+                    acc = __builtin_fmaf(__uint_as_float(wa << 16), bf_at(x[0], e), acc);
+                    acc = __builtin_fmaf(__uint_as_float(wa & 0xffff0000u), bf_at(x[1], e), acc);
+                    acc = __builtin_fmaf(__uint_as_float(wb << 16), bf_at(x[2], e), acc);
+                    acc = __builtin_fmaf(__uint_as_float(wb & 0xffff0000u), bf_at(x[3], e), acc);
+                    s2[k] = bfround(acc * fast_sigmoid(acc));
+                    if (seg == 0) ssq = __builtin_fmaf(s2[k], s2[k], ssq);
+                    if (seg == 1) ssk = __builtin_fmaf(s2[k], s2[k], ssk);
+                    if (seg == 2) VT[(32 * g + 8 * p + e) * LD64 + R] = f2h(s2[k]);
                 }
-                // Rows past the request's end are not masked: their beta is zero, which removes them from L, W, U
-                // and the state update, and their outputs are never stored.
-                const uint16_t qb = f2bf(aq * fast_sigmoid(aq)), kb = f2bf(ak * fast_sigmoid(ak));
-                const float sv = bfround(av * fast_sigmoid(av));
-                qr[i] = bf2f(qb);
-                kr[i] = bf2f(kb);
-                rawq[(lr0 + i) * LD128 + d] = qb;
-                rawk[(lr0 + i) * LD128 + d] = kb;
-                const uint32_t hv = f2h(sv);        // a bf16 value is exact in fp16 (but for values below 2^-14)
-                if (i & 1) vpack[i / 2] |= hv << 16; else vpack[i / 2] = hv;
+                const uint32_t pair = (__float_as_uint(s2[0]) >> 16) | (__float_as_uint(s2[1]) & 0xffff0000u);
+                if (seg == 0) qr[4 * p + e2] = pair;
+                if (seg == 1) kr[4 * p + e2] = pair;
             }
-            uint4* dst = reinterpret_cast<uint4*>(VT + d * LD64 + SUB * a);
-            dst[0] = make_uint4(vpack[0], vpack[1], vpack[2], vpack[3]);
-            dst[1] = make_uint4(vpack[4], vpack[5], vpack[6], vpack[7]);
+            if (it + 1 < 12) {
+#pragma unroll
+                for (int tap = 0; tap < TAPS; ++tap) x[tap] = xn[tap];
+            }
+            __builtin_amdgcn_sched_barrier(0);        // one piece of loads in flight, not all twelve
         }
-        __syncthreads();
-        // L2 norms of the half's 32 rows of q and k: four lanes per (row, q|k), 32 channels each
-        {
-            const int task = t >> 2, part = t & 3;
-            const int row = task & 31, which = task >> 5;
-            const uint16_t* src = (which == 0 ? rawq : rawk) + row * LD128 + 32 * part;
-            float ss = 0.0f;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint4 u = *reinterpret_cast<const uint4*>(src + 8 * j);
-                const uint32_t wds[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float lo = __uint_as_float(wds[e] << 16), hi = __uint_as_float(wds[e] & 0xffff0000u);
-                    ss = __builtin_fmaf(lo, lo, ss);
-                    ss = __builtin_fmaf(hi, hi, ss);
-                }
-            }
-            ss = ss + lane_xor16<1>(ss);
-            ss = ss + lane_xor16<2>(ss);
-            if (part == 0) {
-                float inv = __builtin_amdgcn_rsqf(ss + 1e-6f);
-                if (which == 0) inv *= 0.08838834764831845f;   // 128^-0.5
-                inv_s[which * CH + 32 * h2 + row] = inv;
-            }
-        }
-        __syncthreads();
-        // operands of this lane's 16 rows
-        {
-            float* KrD = reinterpret_cast<float*>(smem + I_DIAG);
-            float* QrD = KrD + 32 * LDG;
-            float* KcD = QrD + 32 * LDG;
-            uint16_t* KR2 = reinterpret_cast<uint16_t*>(smem + I_R2);
-            uint16_t* QR2 = KR2 + 16 * LD128;
-            uint16_t* KC2 = QR2 + 16 * LD128;
-            uint16_t* KR1 = reinterpret_cast<uint16_t*>(smem + I_R1);
-            uint16_t* QR1 = KR1 + 32 * LD128;
-            const float g0 = cg[h2][0];
-            const float eneg0 = fast_exp(-g0);                 // e^{-g of the sub-chunk's first row}
-            const float ep_last = fast_exp(cg[h2][SUB - 1] - g0);
-            const float eB = fast_exp(Bp[a]);                   // e^{G before this sub-chunk}
-            const float eSuf = fast_exp(Bp[4] - Bp[a + 1]);     // e^{G_last - G at this sub-chunk's end}
-            // around the chunk's middle: columns of sub-chunk 0 still cross sub-chunk 1, rows of 3 crossed 2
-            const float eMid = (a == 0) ? fast_exp(tot[1 * DK + d]) : (a == 3 ? fast_exp(tot[2 * DK + d]) : 1.0f);
-            uint32_t kepack[SUB / 2], kgpack[SUB / 2];
-            float kinv[SUB], qinv[SUB];               // read before the stores below (same memory, see the conv)
-#pragma unroll
-            for (int i = 0; i < SUB; ++i) {
-                kinv[i] = inv_s[CH + SUB * a + i];
-                qinv[i] = inv_s[SUB * a + i];
-            }
-#pragma unroll
-            for (int i = 0; i < SUB; ++i) {
-                const int R = SUB * a + i;
-                const float kh = kr[i] * kinv[i], qh = qr[i] * qinv[i];
-                const float e1 = fast_exp(cg[h2][i]);           // e^{G_i - G at the sub-chunk's start}
-                const float ep = e1 * eneg0;                    // e^{G_i - G_first}
-                const float rp = fast_rcp(ep);                  // e^{G_first - G_i}, up to e^87
-                const float col2 = ep_last * rp;                // e^{G at the sub-chunk's end - G_i}
-                const int lr = lr0 + i;
-                KrD[lr * LDG + d] = kh * ep;
-                QrD[lr * LDG + d] = qh * ep;
-                KcD[lr * LDG + d] = kh * rp;
-                if (s == 1) {
-                    KR2[i * LD128 + d] = f2h(kh * e1);
-                    QR2[i * LD128 + d] = f2h(qh * e1);
-                } else {
-                    KC2[i * LD128 + d] = f2h(kh * col2);
-                }
-                if (h2 == 0) {
-                    KC1[lr * LD128 + d] = f2h(kh * col2 * eMid);
-                } else {
-                    KR1[lr * LD128 + d] = f2h(kh * e1 * eMid);
-                    QR1[lr * LD128 + d] = f2h(qh * e1 * eMid);
-                }
-                const uint32_t ke = f2h(kh * e1 * eB), kg = f2h(kh * col2 * eSuf);
-                if (i & 1) { kepack[i / 2] |= ke << 16; kgpack[i / 2] |= kg << 16; }
-                else { kepack[i / 2] = ke; kgpack[i / 2] = kg; }
-                reinterpret_cast<uint16_t*>(wsc + WS_QG)[panel_index(CH, R, d)] = f2h(qh * e1 * eB);
-            }
-            uint4* kd = reinterpret_cast<uint4*>(keT + d * LD64 + SUB * a);
-            kd[0] = make_uint4(kepack[0], kepack[1], kepack[2], kepack[3]);
-            kd[1] = make_uint4(kepack[4], kepack[5], kepack[6], kepack[7]);
-            uint4* gd = reinterpret_cast<uint4*>(wsc + WS_KGT + panel_index(DK, d, SUB * a) * 2);
-            gd[0] = make_uint4(kgpack[0], kgpack[1], kgpack[2], kgpack[3]);
-            gd[1] = make_uint4(kgpack[4], kgpack[5], kgpack[6], kgpack[7]);
-        }
-        __syncthreads();
-        // the half's blocks of L and M on the matrix cores
-        {
-            const float* KrD = reinterpret_cast<const float*>(smem + I_DIAG);
-            const float* QrD = KrD + 32 * LDG;
-            const float* KcD = QrD + 32 * LDG;
-            const uint16_t* KR2 = reinterpret_cast<const uint16_t*>(smem + I_R2);
-            const uint16_t* QR2 = KR2 + 16 * LD128;
-            const uint16_t* KC2 = QR2 + 16 * LD128;
-            const uint16_t* KR1 = reinterpret_cast<const uint16_t*>(smem + I_R1);
-            const uint16_t* QR1 = KR1 + 32 * LD128;
-            uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
-            const int rl = 4 * (lane >> 4), cl = lane & 15;   // this lane's rows rl..rl+3 and column cl of a tile
-            // Store a finished tile at block (rb, cb). L = beta_i * acc: a diagonal block (strictly lower) in f32 for
-            // the inversion, a block below the diagonal negated in fp16 as an MFMA operand of the block solve.
-            // M (lower with the diagonal) goes to the workspace.
-            auto put_L = [&](f32x4 acc, int rb, int cb) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int li = rl + r, gi = SUB * rb + li, gj = SUB * cb + cl;
-                    const float v = beta_s[gi] * acc[r];
-                    if (rb == cb) {
-                        Ld[(SUB * rb + li) * LDD + cl] = cl < li ? v : 0.0f;
-                        Ln[gi * LD64 + gj] = 0;
-                    } else {
-                        Ln[gi * LD64 + gj] = f2h(-v);
-                    }
-                }
-            };
-            auto put_M = [&](f32x4 acc, int rb, int cb) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int gi = SUB * rb + rl + r, gj = SUB * cb + cl;
-                    Mg[panel_index(CH, gi, gj)] = f2h((rb != cb || gj <= gi) ? acc[r] : 0.0f);
-                }
-            };
-            const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-            // diagonal blocks: waves 0, 1 take L of sub-chunks 2 h2, 2 h2 + 1; waves 2, 3 take M
-            {
-                const int sub = wave & 1, blk = 2 * h2 + sub;
-                if (wave < 2) put_L(tile_f32(KrD, SUB * sub, KcD, SUB * sub, lane, zero), blk, blk);
-                else put_M(tile_f32(QrD, SUB * sub, KcD, SUB * sub, lane, zero), blk, blk);
-            }
-            // the block between the half's two sub-chunks
-            if (wave == 0) put_L(tile_f16(KR2, 0, LD128, KC2, 0, LD128, DK, lane, zero), 2 * h2 + 1, 2 * h2);
-            if (wave == 2) put_M(tile_f16(QR2, 0, LD128, KC2, 0, LD128, DK, lane, zero), 2 * h2 + 1, 2 * h2);
-            // rows of the second half against columns of the first
-            if (h2 == 1) {
-#pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    const int idx = 2 * wave + q;              // 0..3: L tiles, 4..7: M tiles
-                    const int ra = (idx >> 1) & 1, cb = idx & 1;
-                    if (idx < 4) put_L(tile_f16(KR1, SUB * ra, LD128, KC1, SUB * cb, LD128, DK, lane, zero), 2 + ra, cb);
-                    else put_M(tile_f16(QR1, SUB * ra, LD128, KC1, SUB * cb, LD128, DK, lane, zero), 2 + ra, cb);
-                }
-            }
-        }
-        __syncthreads();
     }
+    // L2 norms: the four lanes of a row hold 32 channels each
+    ssq += __shfl_xor(ssq, 16, 64);
+    ssq += __shfl_xor(ssq, 32, 64);
+    ssk += __shfl_xor(ssk, 16, 64);
+    ssk += __shfl_xor(ssk, 32, 64);
+    const float qinv = __builtin_amdgcn_rsqf(ssq + 1e-6f) * 0.08838834764831845f;   // 128^-0.5
+    const float kinv = __builtin_amdgcn_rsqf(ssk + 1e-6f);
+    // ---- gates: the cumulative log decay of the lane's row inside its sub-chunk, per channel
+    float G[32];
+    {
+        // a row past the end reads the last real row and counts as g = 0
+        const bf16_t* arow = A + (rr.row0 + r0 + min(R, n - 1)) * a_stride + h * DK + 32 * g;
+        const uint32_t keep = R < n ? 0xffffffffu : 0u;
+        u32x4 av[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            if constexpr (VEC) av[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(arow + 8 * p));
+            else av[p] = load8<false>(arow + 8 * p);
+        }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const f32x4 d0 = *reinterpret_cast<const f32x4*>(dtb_s + 32 * g + 8 * p);
+            const f32x4 d1 = *reinterpret_cast<const f32x4*>(dtb_s + 32 * g + 8 * p + 4);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float dtb = e < 4 ? d0[e] : d1[e - 4];
+                const float gv = lower * fast_sigmoid(rate * (bf_at(av[p], e) + dtb));
+                float x = __uint_as_float(__float_as_uint(gv) & keep);
+                x += row_shr<1>(x);               // inclusive scan over the sixteen rows
+                x += row_shr<2>(x);
+                x += row_shr<4>(x);
+                x += row_shr<8>(x);
+                G[8 * p + e] = x;
+            }
+        }
+        if (i == SUB - 1) {
+#pragma unroll
+            for (int p = 0; p < 8; ++p)
+                *reinterpret_cast<f32x4*>(tot + wave * DK + 32 * g + 4 * p) = f32x4{G[4 * p], G[4 * p + 1], G[4 * p + 2], G[4 * p + 3]};
+        }
+    }
+    if (t < CH) {
+        const bf16_t b_raw = t < n ? P[(rr.row0 + r0 + t) * p_stride + b_off + h] : (bf16_t)0;
+        beta_s[t] = t < n ? bfround(fast_sigmoid(bf2f(b_raw))) : 0.0f;
+    }
+    __syncthreads();
+    // the factors between sub-chunks, one channel per lane; e^{G_last} goes to the workspace
+    {
+        const int d = t & (DK - 1);
+        const float t0 = tot[d], t1 = tot[DK + d], t2 = tot[2 * DK + d], t3 = tot[3 * DK + d];
+        if (t < DK) {
+            fac[0 * DK + d] = 1.0f;
+            fac[1 * DK + d] = fast_exp(t0);
+            fac[2 * DK + d] = fast_exp(t0 + t1);
+            fac[3 * DK + d] = fast_exp(t0 + t1 + t2);
+            reinterpret_cast<float*>(wsc + WS_E)[d] = fast_exp(t0 + t1 + t2 + t3);
+            fac[4 * DK + d] = fast_exp(t1 + t2 + t3);
+            fac[5 * DK + d] = fast_exp(t2 + t3);
+        } else {
+            fac[6 * DK + d] = fast_exp(t3);
+            fac[7 * DK + d] = 1.0f;
+            fac[factor_index(1, 0) * DK + d] = 1.0f;
+            fac[factor_index(2, 0) * DK + d] = fast_exp(t1);
+            fac[factor_index(2, 1) * DK + d] = 1.0f;
+            fac[factor_index(3, 0) * DK + d] = fast_exp(t1 + t2);
+            fac[factor_index(3, 1) * DK + d] = fast_exp(t2);
+            fac[factor_index(3, 2) * DK + d] = 1.0f;
+        }
+    }
+
+    __syncthreads();                              // the factors are in place
+
+    // ---- operands. Per element: e1 = e^{G_i} (from the sub-chunk's start), ep = e^{G_i - G_0} and its reciprocal
+    // (G_0: the sub-chunk's first row, so that fifteen rows of decay bound the exponent), col2 = e^{G_15 - G_i}.
+    // The diagonal tiles of L and M take k ep, q ep (rows) and k / ep (columns) straight from registers, four
+    // channels per f32 MFMA (one per lane group).
+    const int rl = 4 * (lane >> 4), cl = lane & 15;   // an accumulator holds rows rl..rl+3 of column cl of a tile
+    uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
+    // Store a finished tile at block (rb, cb). L = beta_i * acc: a diagonal block (strictly lower) in f32 for the
+    // inversion, a block below the diagonal negated in fp16 as an MFMA operand of the block solve. M (lower with
+    // the diagonal) goes to the workspace.
+    auto put_L = [&](f32x4 acc, int rb, int cb) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int li = rl + r, gi = SUB * rb + li, gj = SUB * cb + cl;
+            const float v = beta_s[gi] * acc[r];
+            if (rb == cb) {
+                Ld[(SUB * rb + li) * LDD + cl] = cl < li ? v : 0.0f;
+                Ln[gi * LD64 + gj] = 0;
+            } else {
+                Ln[gi * LD64 + gj] = f2h(-v);
+            }
+        }
+    };
+    auto put_M = [&](f32x4 acc, int rb, int cb) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int gi = SUB * rb + rl + r, gj = SUB * cb + cl;
+            Mg[panel_index(CH, gi, gj)] = f2h((rb != cb || gj <= gi) ? acc[r] : 0.0f);
+        }
+    };
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    float ke1[32], qe1[32];                       // k e^{G_i}, q e^{G_i}: the row side of the tiles left of the diagonal
+    {
+        f32x4 accL = zero, accM = zero;
+        uint16_t* kgT = reinterpret_cast<uint16_t*>(wsc + WS_KGT);
+        const float* eB = fac + wave * DK + 32 * g;
+        const float* eSuf = fac + (4 + wave) * DK + 32 * g;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const f32x4 b0 = *reinterpret_cast<const f32x4*>(eB + 8 * p), b1 = *reinterpret_cast<const f32x4*>(eB + 8 * p + 4);
+            const f32x4 s0 = *reinterpret_cast<const f32x4*>(eSuf + 8 * p), s1 = *reinterpret_cast<const f32x4*>(eSuf + 8 * p + 4);
+            float qg[8], kc[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int ch = 8 * p + e;
+                const float Gi = G[ch];
+                const float G0 = row_lane<0>(Gi);
+                const float e1 = fast_exp(Gi);
+                const float ep = fast_exp(Gi - G0);
+                const float rp = fast_rcp(ep);                  // e^{G_0 - G_i}, up to e^87
+                const float col2 = row_lane<SUB - 1>(ep) * rp;  // e^{G_15 - G_i}
+                const float kraw = (ch & 1) ? __uint_as_float(kr[ch >> 1] & 0xffff0000u) : __uint_as_float(kr[ch >> 1] << 16);
+                const float qraw = (ch & 1) ? __uint_as_float(qr[ch >> 1] & 0xffff0000u) : __uint_as_float(qr[ch >> 1] << 16);
+                const float kh = kraw * kinv, qh = qraw * qinv;
+                const float kcd = kh * rp;
+                accL = __builtin_amdgcn_mfma_f32_16x16x4f32(kh * ep, kcd, accL, 0, 0, 0);
+                accM = __builtin_amdgcn_mfma_f32_16x16x4f32(qh * ep, kcd, accM, 0, 0, 0);
+                ke1[ch] = kh * e1;
+                qe1[ch] = qh * e1;
+                const float fb = e < 4 ? b0[e] : b1[e - 4], fs = e < 4 ? s0[e] : s1[e - 4];
+                keT[(32 * g + ch) * LD64 + R] = f2h(ke1[ch] * fb);
+                kgT[panel_index(DK, 32 * g + ch, R)] = f2h(kh * col2 * fs);
+                qg[e] = qe1[ch] * fb;
+                kc[e] = kh * col2;
+            }
+            *reinterpret_cast<u32x4*>(wsc + WS_QG + panel_index(CH, R, 32 * g + 8 * p) * 2) =
+                u32x4{pack_h2(qg[0], qg[1]), pack_h2(qg[2], qg[3]), pack_h2(qg[4], qg[5]), pack_h2(qg[6], qg[7])};
+            if (wave < 3)
+                *reinterpret_cast<u32x4*>(KcE + (wave * SUB + i) * LD128 + 32 * g + 8 * p) =
+                    u32x4{pack_h2(kc[0], kc[1]), pack_h2(kc[2], kc[3]), pack_h2(kc[4], kc[5]), pack_h2(kc[6], kc[7])};
+        }
+        put_L(accL, wave, wave);
+        put_M(accM, wave, wave);
+    }
+    __syncthreads();                              // the column operands of every sub-chunk are in place
+    // tiles left of the diagonal: rows of sub-chunk `wave` against the columns of sub-chunk cb. In MFMA step s lane
+    // group g supplies channels 32 g + 8 s .. + 7 on both sides (which k a lane supplies is free as long as both
+    // operands agree).
+#pragma unroll 1
+    for (int cb = 0; cb < wave; ++cb) {
+        const float* df = fac + factor_index(wave, cb) * DK + 32 * g;
+        const uint16_t* kcol = KcE + (cb * SUB + i) * LD128 + 32 * g;
+        f32x4 accL = zero, accM = zero;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const f32x4 d0 = *reinterpret_cast<const f32x4*>(df + 8 * s), d1 = *reinterpret_cast<const f32x4*>(df + 8 * s + 4);
+            const uint4 bcol = *reinterpret_cast<const uint4*>(kcol + 8 * s);
+            float ak[8], aq[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float f = e < 4 ? d0[e] : d1[e - 4];
+                ak[e] = ke1[8 * s + e] * f;
+                aq[e] = qe1[8 * s + e] * f;
+            }
+            const uint4 ka = make_uint4(pack_h2(ak[0], ak[1]), pack_h2(ak[2], ak[3]), pack_h2(ak[4], ak[5]), pack_h2(ak[6], ak[7]));
+            const uint4 qa = make_uint4(pack_h2(aq[0], aq[1]), pack_h2(aq[2], aq[3]), pack_h2(aq[4], aq[5]), pack_h2(aq[6], aq[7]));
+            accL = mfma_f16(ka, bcol, accL);
+            accM = mfma_f16(qa, bcol, accM);
+        }
+        put_L(accL, wave, cb);
+        put_M(accM, wave, cb);
+    }
+    __syncthreads();                              // L is complete; the factors and column operands are dead
     // M and -L above the block diagonal are zero: blocks (0,1), (0,2), (0,3), (1,2), (1,3), (2,3)
     {
         uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
@@ -619,7 +528,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         *reinterpret_cast<uint4*>(wsc + WS_UT + (v * CH + 8 * piece) * 2) =
             *reinterpret_cast<const uint4*>(VT + v * LD64 + 8 * piece);
     }
-    __syncthreads();                              // the next chunk reuses every LDS region
+    __syncthreads();                              // the next chunk's conv writes VT before its first barrier
     }
 }
 
@@ -966,8 +875,10 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
     hipStream_t st = (hipStream_t)stream;
     static bool attr_set = false;
     if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&intra_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                INTRA_LDS) != hipSuccess ||
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&intra_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, INTRA_LDS) != hipSuccess ||
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&intra_kernel<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, INTRA_LDS) != hipSuccess ||
             hipFuncSetAttribute(reinterpret_cast<const void*>(&inter_kernel<float>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, INTER_LDS) != hipSuccess ||
             hipFuncSetAttribute(reinterpret_cast<const void*>(&inter_kernel<bf16_t>),
@@ -985,9 +896,15 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
     const int step = (int)chunks * CH;
     for (int sub0 = 0; sub0 == 0 || sub0 < max_rows; sub0 += step) {
         if (max_rows > 0) {
-            intra_kernel<<<dim3((unsigned)((chunks + INTRA_CPW - 1) / INTRA_CPW), heads, batch), THREADS, INTRA_LDS, st>>>(
-                heads, cu_rows, rows1, sub0, (int)chunks, bfp(p), p_stride, b_off, bfp(a), a_stride, bfp(conv), coff,
-                bfp(conv_w), a_log, dt_bias, lower, vec, ws);
+            const dim3 grid((unsigned)((chunks + INTRA_CPW - 1) / INTRA_CPW), heads, batch);
+            if (vec)
+                intra_kernel<true><<<grid, THREADS, INTRA_LDS, st>>>(heads, cu_rows, rows1, sub0, (int)chunks, bfp(p),
+                                                                     p_stride, b_off, bfp(a), a_stride, bfp(conv), coff,
+                                                                     bfp(conv_w), a_log, dt_bias, lower, ws);
+            else
+                intra_kernel<false><<<grid, THREADS, INTRA_LDS, st>>>(heads, cu_rows, rows1, sub0, (int)chunks, bfp(p),
+                                                                      p_stride, b_off, bfp(a), a_stride, bfp(conv), coff,
+                                                                      bfp(conv_w), a_log, dt_bias, lower, ws);
             const int rc = (int)hipGetLastError();
             if (rc != 0) return rc;
         }
