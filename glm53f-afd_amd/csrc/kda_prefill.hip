@@ -17,8 +17,8 @@
 //
 // Kernels per pass: intra_kernel (one workgroup per chunk, head, request: prologue + L, M, T, W, U, Qg, Kg into
 // the workspace), inter_kernel (one workgroup per head, value-column block, request: the state in MFMA
-// accumulators across the chunks of the pass), then norm_kernel (gated RMSNorm in place) and
-// conv_advance_kernel.
+// accumulators across the chunks of the pass), then norm_kernel (gated RMSNorm in place, and the conv windows'
+// advance).
 
 #include "kda_common.h"
 
@@ -69,12 +69,12 @@ __device__ __forceinline__ f32x4 mfma_f16(uint4 a, uint4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
-// LDS map of intra_kernel, bytes. 75.5 KB: two workgroups share a CU.
+// LDS map of intra_kernel, bytes. 78.5 KB: two workgroups share a CU.
 constexpr int LDD = SUB + 4;                      // f32 row stride of a diagonal block of L (16-byte multiple)
 constexpr int LDT = 40, LDZ = 24;                 // 16-bit row strides of TT and Z (16-byte multiples)
 constexpr int NFAC = 14;                          // per-channel factors between sub-chunks (see factor_index)
-constexpr int I_CW = 0;                           // bf16 [q | k | v][128 channels][4 taps]: the head's conv weights
-constexpr int I_DTB = I_CW + 3 * DK * TAPS * 2;   // f32 [128]: the head's dt_bias
+constexpr int I_CW = 0;                           // f32 [q | k | v][128 channels][4 taps]: the head's conv weights
+constexpr int I_DTB = I_CW + 3 * DK * TAPS * 4;   // f32 [128]: the head's dt_bias
 constexpr int I_TOT = I_DTB + DK * 4;             // f32 [4][128]: log-decay totals of the sub-chunks
 constexpr int I_BETA = I_TOT + 4 * DK * 4;        // f32 [64]
 constexpr int I_KET = I_BETA + CH * 4;            // fp16 [128 keys][LD64]: k e^G, transposed
@@ -100,6 +100,14 @@ __device__ __forceinline__ int factor_index(int a, int b) { return 8 + a * (a - 
 template <int N>
 __device__ __forceinline__ float row_shr(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x110 + N, 0xf, 0xf, false));
+}
+template <int N>
+__device__ __forceinline__ uint32_t row_shl_u(uint32_t x) {   // the value n lanes above (0 where there is none)
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x100 + N, 0xf, 0xf, false);
+}
+template <int N>
+__device__ __forceinline__ uint32_t row_shr_keep(uint32_t keep, uint32_t x) {   // x from n lanes below, else `keep`
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)keep, (int)x, 0x110 + N, 0xf, 0xf, false);
 }
 template <int N>
 __device__ __forceinline__ float row_lane(float x) {
@@ -143,7 +151,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     const long long C = 3LL * H * DK;
     const bf16_t* cs = conv + (conv_off != nullptr ? conv_off[b] : 0);
 
-    uint2* cw_s = reinterpret_cast<uint2*>(smem + I_CW);            // [3 * 128] channels, four taps each
+    f32x4* cw_s = reinterpret_cast<f32x4*>(smem + I_CW);            // [3 * 128] channels, four taps each
     float* dtb_s = reinterpret_cast<float*>(smem + I_DTB);
     float* tot = reinterpret_cast<float*>(smem + I_TOT);
     float* beta_s = reinterpret_cast<float*>(smem + I_BETA);
@@ -156,12 +164,26 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
 
     // the head's conv weights and dt_bias, once (the first barrier of the chunk loop publishes them... they are
     // read before it, so one barrier here)
-    for (int e = t; e < 3 * DK; e += THREADS)
-        cw_s[e] = *reinterpret_cast<const uint2*>(cw + ((size_t)(e >> 7) * H * DK + (size_t)h * DK + (e & (DK - 1))) * TAPS);
+    for (int e = t; e < 3 * DK; e += THREADS) {
+        const uint2 w4 = *reinterpret_cast<const uint2*>(cw + ((size_t)(e >> 7) * H * DK + (size_t)h * DK + (e & (DK - 1))) * TAPS);
+        cw_s[e] = f32x4{__uint_as_float(w4.x << 16), __uint_as_float(w4.x & 0xffff0000u), __uint_as_float(w4.y << 16),
+                        __uint_as_float(w4.y & 0xffff0000u)};
+    }
     if (t < DK) dtb_s[t] = dt_bias[h * DK + t];
     const float rate = fast_exp(a_log[h]);
     __syncthreads();
 
+    // Every lane's own row of q | k | v (twelve 128-bit pieces: its 32 channels of each) is requested a chunk
+    // ahead: for the first chunk here, for the others while the chunk before is in its block solve. A row past the
+    // end is replaced by the last real row (it only feeds rows past the end).
+    u32x4 own[12];
+    auto load_own = [&](int first_row) {
+        const int rel = min(first_row + (int)(t & 15) + SUB * (int)(t >> 6), rr.rows - 1);
+        const bf16_t* src = P + (rr.row0 + rel) * p_stride + h * DK + 32 * ((t >> 4) & 3);
+#pragma unroll
+        for (int it = 0; it < 12; ++it) own[it] = load8<VEC>(src + (long long)(it >> 2) * H * DK + 8 * (it & 3));
+    };
+    load_own(sub0 + c_first * CH);
 #pragma unroll 1
     for (int c = c_first; c < min(chunks, c_first + INTRA_CPW); ++c) {
     // t, and what derives from it, are re-made for every chunk from a value the optimizer cannot see through:
@@ -181,52 +203,52 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     uint32_t qr[16], kr[16];                      // bf16 pairs: the conv outputs are bf16 values
     float ssq = 0.0f, ssk = 0.0f;
     {
-        // a tap row past the end only feeds rows past the end: it reads the last real row instead
-        const bf16_t* rowp[TAPS];
+        // The conv's tap 3 is the lane's own row; the three rows before it are the own rows of the lanes below, a
+        // DPP shift away. Lanes 0..2 of a sub-chunk also need the three rows before the sub-chunk (the conv window,
+        // for the request's first rows): lane j < 3 loads row 16 w - 3 + j as its `halo`, zero in the other lanes.
+        u32x4 halo[12];
+        {
 #pragma unroll
-        for (int tap = 0; tap < TAPS; ++tap) {
-            const int rel = min(r0 + R - WINDOW + tap, rr.rows - 1);
-            rowp[tap] = (rel < 0 ? cs + (long long)(rel + WINDOW) * C : P + (rr.row0 + rel) * p_stride) + h * DK + 32 * g;
+            for (int it = 0; it < 12; ++it) halo[it] = u32x4{0u, 0u, 0u, 0u};
+            if (i < WINDOW) {
+                const int hrel = min(r0 + SUB * wave - WINDOW + i, rr.rows - 1);
+                const bf16_t* hsrc = (hrel < 0 ? cs + (long long)(hrel + WINDOW) * C : P + (rr.row0 + hrel) * p_stride) +
+                                     h * DK + 32 * g;
+#pragma unroll
+                for (int it = 0; it < 12; ++it) halo[it] = load8<VEC>(hsrc + (long long)(it >> 2) * H * DK + 8 * (it & 3));
+            }
         }
-        u32x4 x[TAPS], xn[TAPS];
-#pragma unroll
-        for (int tap = 0; tap < TAPS; ++tap) x[tap] = load8<VEC>(rowp[tap]);
 #pragma unroll
         for (int it = 0; it < 12; ++it) {
             const int seg = it >> 2, p = it & 3;
-            if (it + 1 < 12) {
-                const int seg1 = (it + 1) >> 2, p1 = (it + 1) & 3;
 #pragma unroll
-                for (int tap = 0; tap < TAPS; ++tap)
-                    xn[tap] = load8<VEC>(rowp[tap] + (long long)seg1 * H * DK + 8 * p1);
-            }
-#pragma unroll
-            for (int e2 = 0; e2 < 4; ++e2) {      // two channels per 128-bit piece of weights
-                const u32x4 w2 = *reinterpret_cast<const u32x4*>(cw_s + seg * DK + 32 * g + 8 * p + 2 * e2);
+            for (int d = 0; d < 4; ++d) {         // a 32-bit word holds two channels
+                // taps 0..2 are the rows above: the own rows of the lanes below, or (lanes 0..2) halo rows, which a
+                // DPP move leaves in place where it has no source lane
+                const uint32_t x3 = own[it][d], hl = halo[it][d];
+                const uint32_t x0 = row_shr_keep<3>(hl, x3);
+                const uint32_t x1 = row_shr_keep<2>(row_shl_u<1>(hl), x3);
+                const uint32_t x2 = row_shr_keep<1>(row_shl_u<2>(hl), x3);
                 float s2[2];
 #pragma unroll
                 for (int k = 0; k < 2; ++k) {
-                    const int e = 2 * e2 + k;
-                    const uint32_t wa = w2[2 * k], wb = w2[2 * k + 1];
-                    float acc = 0.0f;
-                    acc = __builtin_fmaf(__uint_as_float(wa << 16), bf_at(x[0], e), acc);
-                    acc = __builtin_fmaf(__uint_as_float(wa & 0xffff0000u), bf_at(x[1], e), acc);
-                    acc = __builtin_fmaf(__uint_as_float(wb << 16), bf_at(x[2], e), acc);
-                    acc = __builtin_fmaf(__uint_as_float(wb & 0xffff0000u), bf_at(x[3], e), acc);
-                    s2[k] = bfround(acc * fast_sigmoid(acc));
-                    if (seg == 0) ssq = __builtin_fmaf(s2[k], s2[k], ssq);
-                    if (seg == 1) ssk = __builtin_fmaf(s2[k], s2[k], ssk);
-                    if (seg == 2) VT[(32 * g + 8 * p + e) * LD64 + R] = f2h(s2[k]);
+                    const f32x4 w = cw_s[seg * DK + 32 * g + 8 * p + 2 * d + k];
+                    auto half = [k](uint32_t v) { return k ? __uint_as_float(v & 0xffff0000u) : __uint_as_float(v << 16); };
+                    float acc = w[0] * half(x0);
+                    acc = __builtin_fmaf(w[1], half(x1), acc);
+                    acc = __builtin_fmaf(w[2], half(x2), acc);
+                    acc = __builtin_fmaf(w[3], half(x3), acc);
+                    s2[k] = acc * fast_sigmoid(acc);
                 }
-                const uint32_t pair = (__float_as_uint(s2[0]) >> 16) | (__float_as_uint(s2[1]) & 0xffff0000u);
-                if (seg == 0) qr[4 * p + e2] = pair;
-                if (seg == 1) kr[4 * p + e2] = pair;
+                const uint32_t pair = f2bf2(s2[0], s2[1]);        // the one bf16 rounding
+                const float r0f = __uint_as_float(pair << 16), r1f = __uint_as_float(pair & 0xffff0000u);
+                if (seg == 0) { qr[4 * p + d] = pair; ssq = __builtin_fmaf(r0f, r0f, ssq); ssq = __builtin_fmaf(r1f, r1f, ssq); }
+                if (seg == 1) { kr[4 * p + d] = pair; ssk = __builtin_fmaf(r0f, r0f, ssk); ssk = __builtin_fmaf(r1f, r1f, ssk); }
+                if (seg == 2) {
+                    VT[(32 * g + 8 * p + 2 * d) * LD64 + R] = f2h(r0f);
+                    VT[(32 * g + 8 * p + 2 * d + 1) * LD64 + R] = f2h(r1f);
+                }
             }
-            if (it + 1 < 12) {
-#pragma unroll
-                for (int tap = 0; tap < TAPS; ++tap) x[tap] = xn[tap];
-            }
-            __builtin_amdgcn_sched_barrier(0);        // one piece of loads in flight, not all twelve
         }
     }
     // L2 norms: the four lanes of a row hold 32 channels each
@@ -449,6 +471,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         }
     }
     __syncthreads();
+    load_own(r0 + CH);                            // the next chunk's rows (clamped to the request: never out of bounds)
 
     // ---- W = T' (k e^G) and U = T' v without the blocks of T below the diagonal: block forward substitution on
     // R = [k e^G | v] (64 rows, 256 columns), held transposed in LDS ([column][row]: keT then VT) and solved in
@@ -751,14 +774,34 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
                               accS[mt][nt]);
 }
 
-// The gated RMSNorm over the bf16 read-outs the inter pass left in `out` (reference: kda_prefill.cu:542-570,
+// The call's last launch: the conv windows' advance, and the gated RMSNorm over the bf16 read-outs the inter pass
+// left in `out` (reference: kda_prefill.cu:542-570,
 // cpu.rs:361-376). Sixteen lanes per (row, head), eight values per lane in 128-bit pieces when `wide` (rows of `out`
 // and the gate 16-byte aligned); else a wave per (row, head), two values per lane.
 __global__ void __launch_bounds__(THREADS) norm_kernel(int H, const int32_t* __restrict__ cu_rows, int rows1,
                                                        const bf16_t* __restrict__ G, long long g_stride,
                                                        const bf16_t* __restrict__ norm_w, float eps, bf16_t* out,
-                                                       long long out_stride, int wide) {
+                                                       long long out_stride, int wide, bf16_t* conv,
+                                                       const long long* __restrict__ conv_off,
+                                                       const bf16_t* __restrict__ P, long long p_stride) {
     const RowRange rr = request_rows(cu_rows, blockIdx.y, rows1);
+    // The request's conv window moves past all its rows, in place (reference: kda_prefill.cu:574-590): every channel
+    // is one lane's, which reads its three values before it writes them. Here because this is the call's last
+    // launch: every pass has read the window by now.
+    {
+        const int C = 3 * H * DK;
+        bf16_t* win = conv + (conv_off != nullptr ? conv_off[blockIdx.y] : 0);
+        for (long long c = (long long)blockIdx.x * THREADS + threadIdx.x; c < C; c += (long long)gridDim.x * THREADS) {
+            bf16_t x[WINDOW];
+#pragma unroll
+            for (int j = 0; j < WINDOW; ++j) {
+                const long long src = (long long)rr.rows + j;
+                x[j] = src < WINDOW ? win[src * C + c] : P[(rr.row0 + src - WINDOW) * p_stride + c];
+            }
+#pragma unroll
+            for (int j = 0; j < WINDOW; ++j) win[(long long)j * C + c] = x[j];
+        }
+    }
     const long long tasks = (long long)rr.rows * H;
     const int lane = threadIdx.x & 63;
     if (wide) {
@@ -818,25 +861,6 @@ __global__ void __launch_bounds__(THREADS) norm_kernel(int H, const int32_t* __r
         const float g0 = __uint_as_float(gg << 16), g1 = __uint_as_float(gg & 0xffff0000u);
         o[lane] = f2bf2(w0 * (y0 * rinv) * fast_sigmoid(g0), w1 * (y1 * rinv) * fast_sigmoid(g1));
     }
-}
-
-// Advance each request's conv window past all its rows, in place (reference: kda_prefill.cu:574-590): each lane
-// reads its three values before writing them.
-__global__ void conv_advance_kernel(int C, const int32_t* __restrict__ cu_rows, int rows1, bf16_t* conv,
-                                    const long long* __restrict__ conv_off, const bf16_t* __restrict__ P,
-                                    long long p_stride) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= C) return;
-    const RowRange rr = request_rows(cu_rows, blockIdx.y, rows1);
-    bf16_t* win = conv + (conv_off != nullptr ? conv_off[blockIdx.y] : 0);
-    bf16_t x[WINDOW];
-#pragma unroll
-    for (int j = 0; j < WINDOW; ++j) {
-        const long long src = (long long)rr.rows + j;
-        x[j] = src < WINDOW ? win[src * C + c] : P[(rr.row0 + src - WINDOW) * p_stride + c];
-    }
-#pragma unroll
-    for (int j = 0; j < WINDOW; ++j) win[(long long)j * C + c] = x[j];
 }
 
 inline const bf16_t* bfp(const glm53f_bf16* x) { return reinterpret_cast<const bf16_t*>(x); }
@@ -918,14 +942,11 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
     if (max_rows > 0) {
         const int wide = aligned16(out) && aligned16(g) && aligned16(norm_w) && out_stride % 8 == 0 && g_stride % 8 == 0;
         norm_kernel<<<dim3(kNormBlocks, batch), THREADS, 0, st>>>(heads, cu_rows, rows1, bfp(g), g_stride, bfp(norm_w),
-                                                                  eps, bfp(out), out_stride, wide);
-        const int rc = (int)hipGetLastError();
-        if (rc != 0) return rc;
+                                                                  eps, bfp(out), out_stride, wide, bfp(conv), coff,
+                                                                  bfp(p), p_stride);
+        return (int)hipGetLastError();
     }
-    const int C = 3 * heads * DK;
-    conv_advance_kernel<<<dim3((C + 255) / 256, batch), 256, 0, st>>>(C, cu_rows, rows1, bfp(conv), coff, bfp(p),
-                                                                      p_stride);
-    return (int)hipGetLastError();
+    return 0;                                     // no request has rows: the windows stay as they are
 }
 
 }  // namespace
