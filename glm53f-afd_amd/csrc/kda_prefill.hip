@@ -28,6 +28,7 @@ namespace {
 constexpr int CH = 64, SUB = 16, THREADS = 256;
 constexpr int NV = 32;                    // value columns per inter workgroup
 constexpr int VBLOCKS = DV / NV;          // inter workgroups per head
+constexpr int NT = NV / 16;               // 16-column tiles of a workgroup's value block
 
 typedef _Float16 f16_t;
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -73,9 +74,9 @@ __device__ __forceinline__ f32x4 mfma_f16(uint4 a, uint4 b, f32x4 c) {
 constexpr int LDD = SUB + 4;                      // f32 row stride of a diagonal block of L (16-byte multiple)
 constexpr int LDT = 40, LDZ = 24;                 // 16-bit row strides of TT and Z (16-byte multiples)
 constexpr int NFAC = 14;                          // per-channel factors between sub-chunks (see factor_index)
-constexpr int I_CW = 0;                           // f32 [q | k | v][128 channels][4 taps]: the head's conv weights
-constexpr int I_DTB = I_CW + 3 * DK * TAPS * 4;   // f32 [128]: the head's dt_bias
-constexpr int I_TOT = I_DTB + DK * 4;             // f32 [4][128]: log-decay totals of the sub-chunks
+constexpr int I_CW = 0;                           // u32 [q | k | v][128 channels][4 taps]: the head's conv weights
+constexpr int I_DTB = I_CW + 3 * DK * TAPS * 4;   // f32 [128]: the head's dt_bias, times -rate log2(e)
+constexpr int I_TOT = I_DTB + DK * 4;             // f32 [4][128]: log2-decay totals of the sub-chunks
 constexpr int I_BETA = I_TOT + 4 * DK * 4;        // f32 [64]
 constexpr int I_KET = I_BETA + CH * 4;            // fp16 [128 keys][LD64]: k e^G, transposed
 constexpr int I_VT = I_KET + DK * LD64 * 2;       // fp16 [128 values][LD64]: v, transposed
@@ -114,6 +115,12 @@ __device__ __forceinline__ float row_lane(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x150 + N, 0xf, 0xf, false));
 }
 
+// a.lo * b.lo + a.hi * b.hi + c over bf16 pairs (v_dot2c_f32_bf16; within one f32 ulp of the fused form).
+typedef __bf16 hwbf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(hwbf16x2, a), __builtin_bit_cast(hwbf16x2, b), c, false);
+}
+
 // Eight consecutive bf16 from p. With VEC p is 16-byte aligned.
 template <bool VEC>
 __device__ __forceinline__ u32x4 load8(const bf16_t* p) {
@@ -129,7 +136,13 @@ __device__ __forceinline__ u32x4 load8(const bf16_t* p) {
 __device__ __forceinline__ float bf_at(const u32x4 v, int e) {   // element e of eight packed bf16
     return (e & 1) ? __uint_as_float(v[e >> 1] & 0xffff0000u) : __uint_as_float(v[e >> 1] << 16);
 }
-__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) { return (uint32_t)f2h(lo) | ((uint32_t)f2h(hi) << 16); }
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// Two values to fp16 in one instruction (v_cvt_pk_f16_f32, round to nearest even): lo in bits 0..15.
+__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
 
 // Pass 1: the chunks of one head of one request, everything that does not need the state, into their workspace
 // slots. Wave w owns sub-chunk w of a chunk (rows 16 w .. 16 w + 15); in the elementwise phases lane l holds row
@@ -151,7 +164,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     const long long C = 3LL * H * DK;
     const bf16_t* cs = conv + (conv_off != nullptr ? conv_off[b] : 0);
 
-    f32x4* cw_s = reinterpret_cast<f32x4*>(smem + I_CW);            // [3 * 128] channels, four taps each
+    u32x4* cw_s = reinterpret_cast<u32x4*>(smem + I_CW);            // [3 * 128] channels, four taps each
     float* dtb_s = reinterpret_cast<float*>(smem + I_DTB);
     float* tot = reinterpret_cast<float*>(smem + I_TOT);
     float* beta_s = reinterpret_cast<float*>(smem + I_BETA);
@@ -164,13 +177,20 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
 
     // the head's conv weights and dt_bias, once (the first barrier of the chunk loop publishes them... they are
     // read before it, so one barrier here)
+    // A conv weight is stored as the bf16 pair (w, 0) for an even channel and (0, w) for an odd one: the input rows
+    // hold two channels per 32-bit word, and v_dot2c_f32_bf16 of such a word with the pair is w x + acc for the one
+    // channel, with no unpacking.
     for (int e = t; e < 3 * DK; e += THREADS) {
         const uint2 w4 = *reinterpret_cast<const uint2*>(cw + ((size_t)(e >> 7) * H * DK + (size_t)h * DK + (e & (DK - 1))) * TAPS);
-        cw_s[e] = f32x4{__uint_as_float(w4.x << 16), __uint_as_float(w4.x & 0xffff0000u), __uint_as_float(w4.y << 16),
-                        __uint_as_float(w4.y & 0xffff0000u)};
+        const uint32_t w[4] = {w4.x & 0xffffu, w4.x >> 16, w4.y & 0xffffu, w4.y >> 16};
+        const int sh = (e & 1) ? 16 : 0;
+        cw_s[e] = u32x4{w[0] << sh, w[1] << sh, w[2] << sh, w[3] << sh};
     }
-    if (t < DK) dtb_s[t] = dt_bias[h * DK + t];
-    const float rate = fast_exp(a_log[h]);
+    // The gates work in base 2: sigmoid(r (a + dtb)) = 1 / (1 + 2^(c a + c dtb)) with c = -r log2(e), and the log
+    // decays are kept in log2 units (G log2(e)), so that every e^G below is one v_exp_f32.
+    const float gate_c = -fast_exp(a_log[h]) * 1.4426950408889634f;
+    const float lower2 = lower * 1.4426950408889634f;
+    if (t < DK) dtb_s[t] = gate_c * dt_bias[h * DK + t];
     __syncthreads();
 
     // Every lane's own row of q | k | v (twelve 128-bit pieces: its 32 channels of each) is requested a chunk
@@ -232,12 +252,11 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 float s2[2];
 #pragma unroll
                 for (int k = 0; k < 2; ++k) {
-                    const f32x4 w = cw_s[seg * DK + 32 * g + 8 * p + 2 * d + k];
-                    auto half = [k](uint32_t v) { return k ? __uint_as_float(v & 0xffff0000u) : __uint_as_float(v << 16); };
-                    float acc = w[0] * half(x0);
-                    acc = __builtin_fmaf(w[1], half(x1), acc);
-                    acc = __builtin_fmaf(w[2], half(x2), acc);
-                    acc = __builtin_fmaf(w[3], half(x3), acc);
+                    const u32x4 w = cw_s[seg * DK + 32 * g + 8 * p + 2 * d + k];
+                    float acc = dot2_bf16(x0, w[0], 0.0f);
+                    acc = dot2_bf16(x1, w[1], acc);
+                    acc = dot2_bf16(x2, w[2], acc);
+                    acc = dot2_bf16(x3, w[3], acc);
                     s2[k] = acc * fast_sigmoid(acc);
                 }
                 const uint32_t pair = f2bf2(s2[0], s2[1]);        // the one bf16 rounding
@@ -277,7 +296,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float dtb = e < 4 ? d0[e] : d1[e - 4];
-                const float gv = lower * fast_sigmoid(rate * (bf_at(av[p], e) + dtb));
+                const float gv = lower2 * fast_rcp(1.0f + __builtin_amdgcn_exp2f(__builtin_fmaf(gate_c, bf_at(av[p], e), dtb)));
                 float x = __uint_as_float(__float_as_uint(gv) & keep);
                 x += row_shr<1>(x);               // inclusive scan over the sixteen rows
                 x += row_shr<2>(x);
@@ -303,20 +322,20 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         const float t0 = tot[d], t1 = tot[DK + d], t2 = tot[2 * DK + d], t3 = tot[3 * DK + d];
         if (t < DK) {
             fac[0 * DK + d] = 1.0f;
-            fac[1 * DK + d] = fast_exp(t0);
-            fac[2 * DK + d] = fast_exp(t0 + t1);
-            fac[3 * DK + d] = fast_exp(t0 + t1 + t2);
-            reinterpret_cast<float*>(wsc + WS_E)[d] = fast_exp(t0 + t1 + t2 + t3);
-            fac[4 * DK + d] = fast_exp(t1 + t2 + t3);
-            fac[5 * DK + d] = fast_exp(t2 + t3);
+            fac[1 * DK + d] = __builtin_amdgcn_exp2f(t0);
+            fac[2 * DK + d] = __builtin_amdgcn_exp2f(t0 + t1);
+            fac[3 * DK + d] = __builtin_amdgcn_exp2f(t0 + t1 + t2);
+            reinterpret_cast<float*>(wsc + WS_E)[d] = __builtin_amdgcn_exp2f(t0 + t1 + t2 + t3);
+            fac[4 * DK + d] = __builtin_amdgcn_exp2f(t1 + t2 + t3);
+            fac[5 * DK + d] = __builtin_amdgcn_exp2f(t2 + t3);
         } else {
-            fac[6 * DK + d] = fast_exp(t3);
+            fac[6 * DK + d] = __builtin_amdgcn_exp2f(t3);
             fac[7 * DK + d] = 1.0f;
             fac[factor_index(1, 0) * DK + d] = 1.0f;
-            fac[factor_index(2, 0) * DK + d] = fast_exp(t1);
+            fac[factor_index(2, 0) * DK + d] = __builtin_amdgcn_exp2f(t1);
             fac[factor_index(2, 1) * DK + d] = 1.0f;
-            fac[factor_index(3, 0) * DK + d] = fast_exp(t1 + t2);
-            fac[factor_index(3, 1) * DK + d] = fast_exp(t2);
+            fac[factor_index(3, 0) * DK + d] = __builtin_amdgcn_exp2f(t1 + t2);
+            fac[factor_index(3, 1) * DK + d] = __builtin_amdgcn_exp2f(t2);
             fac[factor_index(3, 2) * DK + d] = 1.0f;
         }
     }
@@ -369,8 +388,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 const int ch = 8 * p + e;
                 const float Gi = G[ch];
                 const float G0 = row_lane<0>(Gi);
-                const float e1 = fast_exp(Gi);
-                const float ep = fast_exp(Gi - G0);
+                const float e1 = __builtin_amdgcn_exp2f(Gi);
+                const float ep = __builtin_amdgcn_exp2f(Gi - G0);
                 const float rp = fast_rcp(ep);                  // e^{G_0 - G_i}, up to e^87
                 const float col2 = row_lane<SUB - 1>(ep) * rp;  // e^{G_15 - G_i}
                 const float kraw = (ch & 1) ? __uint_as_float(kr[ch >> 1] & 0xffff0000u) : __uint_as_float(kr[ch >> 1] << 16);
@@ -485,8 +504,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         const int rl = 4 * (lane >> 4), cl = lane & 15;
         const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
         auto pack4 = [](const f32x4 v) {
-            return make_uint2((uint32_t)f2h(v[0]) | ((uint32_t)f2h(v[1]) << 16),
-                              (uint32_t)f2h(v[2]) | ((uint32_t)f2h(v[3]) << 16));
+            return make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
         };
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
@@ -589,7 +607,7 @@ struct InterOperands {
     u32x4 w[4], q[4];                             // rows 16 w + l % 16, keys 32 ks + 8 (l / 16) ..
     u32x4 m[2];                                   // rows 16 w + l % 16, chunk rows 32 ks + 8 (l / 16) ..
     u32x4 k[2][2];                                // keys 32 w + 16 mt + l % 16, chunk rows 32 ks + 8 (l / 16) ..
-    uint2 u[2];                                   // value 16 nt + l % 16, rows 16 w + 4 (l / 16) ..
+    uint2 u[NT];                                   // value 16 nt + l % 16, rows 16 w + 4 (l / 16) ..
     f32x4 e[2];                                   // keys 32 w + 16 mt + 4 (l / 16) ..
 };
 
@@ -617,11 +635,11 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
     uint16_t* Vl = reinterpret_cast<uint16_t*>(smem + N_V);
 
     // the state: accS[mt][nt][r] = S[key 32 w + 16 mt + rl + r][value NV vb + 16 nt + cl]
-    f32x4 accS[2][2];
+    f32x4 accS[2][NT];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
+        for (int nt = 0; nt < NT; ++nt) {
             float v4[4];
             load_state_elem4<S>(state_in + sbase + (long long)(NV * vb + SUB * nt + cl) * DK + 32 * wave + SUB * mt + rl, v4);
             accS[mt][nt] = f32x4{v4[0], v4[1], v4[2], v4[3]};
@@ -640,7 +658,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                               \
         _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                            \
             X_.w[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_W + off_a + 4096 * ks);                              \
-        _Pragma("unroll") for (int nt = 0; nt < 2; ++nt)                                                            \
+        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                            \
             X_.u[nt] = *reinterpret_cast<const uint2*>(src_ + off_u + 2048 * nt);                                    \
     }
 #define KDA_LOAD_QM(X_, C_)                                                                                         \
@@ -665,7 +683,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt) {
+            for (int nt = 0; nt < NT; ++nt) {
                 const uint32_t s0 = (uint32_t)f2h(accS[mt][nt][0]) | ((uint32_t)f2h(accS[mt][nt][1]) << 16);
                 const uint32_t s1 = (uint32_t)f2h(accS[mt][nt][2]) | ((uint32_t)f2h(accS[mt][nt][3]) << 16);
                 *reinterpret_cast<uint2*>(Sl + (SUB * nt + cl) * LD128 + 32 * wave + SUB * mt + rl) = make_uint2(s0, s1);
@@ -681,18 +699,20 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         __syncthreads();      // the state is in LDS; every wave is done with the V' of the chunk before
         const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
         // V' = U - W S: wave w takes rows 16 w .. 16 w + 15
-        uint4 sfrag[2][4];
+        uint4 sfrag[NT][4];
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) sfrag[nt][ks] = frag(Sl, LD128, SUB * nt, 32 * ks, lane);
-        f32x4 accV[2] = {zero, zero};
+        f32x4 accV[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) accV[nt] = zero;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt) accV[nt] = mfma_f16(as_u4(x.w[ks]), sfrag[nt][ks], accV[nt]);
+            for (int nt = 0; nt < NT; ++nt) accV[nt] = mfma_f16(as_u4(x.w[ks]), sfrag[nt][ks], accV[nt]);
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
+        for (int nt = 0; nt < NT; ++nt) {
             const uint2 u = x.u[nt];
             const float v0 = h2f((uint16_t)(u.x & 0xffffu)) - accV[nt][0], v1 = h2f((uint16_t)(u.x >> 16)) - accV[nt][1];
             const float v2 = h2f((uint16_t)(u.y & 0xffffu)) - accV[nt][2], v3 = h2f((uint16_t)(u.y >> 16)) - accV[nt][3];
@@ -703,25 +723,27 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
         KDA_LOAD_W(x, c2)
         __syncthreads();
         // Y = Qg S + M V'
-        uint4 vfrag[2][2];
+        uint4 vfrag[NT][2];
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) vfrag[nt][ks] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
-        f32x4 accY[2] = {zero, zero};
+        f32x4 accY[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) accY[nt] = zero;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt) accY[nt] = mfma_f16(as_u4(x.q[ks]), sfrag[nt][ks], accY[nt]);
+            for (int nt = 0; nt < NT; ++nt) accY[nt] = mfma_f16(as_u4(x.q[ks]), sfrag[nt][ks], accY[nt]);
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt) accY[nt] = mfma_f16(as_u4(x.m[ks]), vfrag[nt][ks], accY[nt]);
+            for (int nt = 0; nt < NT; ++nt) accY[nt] = mfma_f16(as_u4(x.m[ks]), vfrag[nt][ks], accY[nt]);
         KDA_LOAD_QM(x, c2)
         {
             const long long grow0 = rr.row0 + sub0 + c * CH;
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int row = SUB * wave + rl + r;
@@ -733,13 +755,13 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) accS[mt][nt][r] *= x.e[mt][r];
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                for (int nt = 0; nt < 2; ++nt) accS[mt][nt] = mfma_f16(as_u4(x.k[mt][ks]), vfrag[nt][ks], accS[mt][nt]);
+                for (int nt = 0; nt < NT; ++nt) accS[mt][nt] = mfma_f16(as_u4(x.k[mt][ks]), vfrag[nt][ks], accS[mt][nt]);
         }
         KDA_LOAD_KE(x, c2)
         if constexpr (sizeof(S) == 2) {
@@ -747,7 +769,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-                for (int nt = 0; nt < 2; ++nt)
+                for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) accS[mt][nt][r] = bfround(accS[mt][nt][r]);
         }
@@ -769,7 +791,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+        for (int nt = 0; nt < NT; ++nt)
             store_state_elem4(state_out + sbase + (long long)(NV * vb + SUB * nt + cl) * DK + 32 * wave + SUB * mt + rl,
                               accS[mt][nt]);
 }
