@@ -87,7 +87,7 @@ constexpr int I_Z = I_KCE;                        //   later fp16 [16 column til
 constexpr int I_FAC = I_KCE + 3 * SUB * LD128 * 2;  // f32 [NFAC][128]
 constexpr int I_TT = I_FAC;                       //   later fp16 [64][LDT]: row 16 a + i holds [T_aa diag(beta) | T_aa][i][0..32)
 constexpr int INTRA_LDS = I_FAC + NFAC * DK * 4;
-constexpr int INTRA_CPW = 4;                      // consecutive chunks of a head per intra workgroup
+constexpr int INTRA_CPW = 2;                      // consecutive chunks of a head per intra workgroup
 static_assert(16 * SUB * LDZ * 2 <= 3 * SUB * LD128 * 2, "Z fits the region of the column operands");
 static_assert(CH * LDT * 2 <= NFAC * DK * 4, "TT fits the region of the factors");
 static_assert(2 * INTRA_LDS <= 160 * 1024, "two intra workgroups per CU");
@@ -216,6 +216,17 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     if (n <= 0) break;
     const int R = SUB * wave + i;                 // this lane's row inside the chunk
     unsigned char* wsc = ws + (((long long)b * H + h) * chunks + c) * (long long)WS_BYTES;
+    // the row of forget-gate inputs, requested now and used after the conv (a row past the end reads the last real
+    // row and counts as g = 0)
+    u32x4 av[4];
+    {
+        const bf16_t* arow = A + (rr.row0 + r0 + min(R, n - 1)) * a_stride + h * DK + 32 * g;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            if constexpr (VEC) av[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(arow + 8 * p));
+            else av[p] = load8<false>(arow + 8 * p);
+        }
+    }
 
     // ---- conv + SiLU with one bf16 rounding (q, k stay in registers; v goes to VT as fp16, exact but for values
     // below 2^-14), and the sums of squares for the L2 norms. Rows past the request's end are not masked: their
@@ -280,15 +291,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // ---- gates: the cumulative log decay of the lane's row inside its sub-chunk, per channel
     float G[32];
     {
-        // a row past the end reads the last real row and counts as g = 0
-        const bf16_t* arow = A + (rr.row0 + r0 + min(R, n - 1)) * a_stride + h * DK + 32 * g;
-        const uint32_t keep = R < n ? 0xffffffffu : 0u;
-        u32x4 av[4];
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            if constexpr (VEC) av[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(arow + 8 * p));
-            else av[p] = load8<false>(arow + 8 * p);
-        }
+        const uint32_t keep = R < n ? 0xffffffffu : 0u;    // a row past the end counts as g = 0
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const f32x4 d0 = *reinterpret_cast<const f32x4*>(dtb_s + 32 * g + 8 * p);
@@ -490,7 +493,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         }
     }
     __syncthreads();
-    load_own(r0 + CH);                            // the next chunk's rows (clamped to the request: never out of bounds)
+    if (c + 1 < min(chunks, c_first + INTRA_CPW)) load_own(r0 + CH);   // the next chunk's rows
 
     // ---- W = T' (k e^G) and U = T' v without the blocks of T below the diagonal: block forward substitution on
     // R = [k e^G | v] (64 rows, 256 columns), held transposed in LDS ([column][row]: keT then VT) and solved in
