@@ -102,17 +102,19 @@ template <int N>
 __device__ __forceinline__ float row_shr(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x110 + N, 0xf, 0xf, false));
 }
+// The same moves on raw words, in the form that needs no prepared destination (bound_ctrl: lanes without a source
+// read zero): the value n lanes below, and n lanes above.
 template <int N>
-__device__ __forceinline__ uint32_t row_shl_u(uint32_t x) {   // the value n lanes above (0 where there is none)
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x100 + N, 0xf, 0xf, false);
+__device__ __forceinline__ uint32_t row_shr_u(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x110 + N, 0xf, 0xf, true);
 }
 template <int N>
-__device__ __forceinline__ uint32_t row_shr_keep(uint32_t keep, uint32_t x) {   // x from n lanes below, else `keep`
-    return (uint32_t)__builtin_amdgcn_update_dpp((int)keep, (int)x, 0x110 + N, 0xf, 0xf, false);
+__device__ __forceinline__ uint32_t row_shl_u(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x100 + N, 0xf, 0xf, true);
 }
 template <int N>
 __device__ __forceinline__ float row_lane(float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x150 + N, 0xf, 0xf, false));
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x150 + N, 0xf, 0xf, true));
 }
 
 // a.lo * b.lo + a.hi * b.hi + c over bf16 pairs (v_dot2c_f32_bf16; within one f32 ulp of the fused form).
@@ -254,12 +256,12 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             const int seg = it >> 2, p = it & 3;
 #pragma unroll
             for (int d = 0; d < 4; ++d) {         // a 32-bit word holds two channels
-                // taps 0..2 are the rows above: the own rows of the lanes below, or (lanes 0..2) halo rows, which a
-                // DPP move leaves in place where it has no source lane
+                // taps 0..2 are the rows above: the own rows of the lanes below, or (lanes 0..2) halo rows; where one
+                // has nothing (a shifted-in zero, a zero halo) the other has the row
                 const uint32_t x3 = own[it][d], hl = halo[it][d];
-                const uint32_t x0 = row_shr_keep<3>(hl, x3);
-                const uint32_t x1 = row_shr_keep<2>(row_shl_u<1>(hl), x3);
-                const uint32_t x2 = row_shr_keep<1>(row_shl_u<2>(hl), x3);
+                const uint32_t x0 = row_shr_u<3>(x3) | hl;
+                const uint32_t x1 = row_shr_u<2>(x3) | row_shl_u<1>(hl);
+                const uint32_t x2 = row_shr_u<1>(x3) | row_shl_u<2>(hl);
                 float s2[2];
 #pragma unroll
                 for (int k = 0; k < 2; ++k) {
