@@ -34,10 +34,10 @@ from glm53f_kda import DK, DV, HEADS, LAYERS, WINDOW, channels, ffi, state_len
 # script's legs, scaled by the same counters over the 1 GiB copy of --only copy: x2.00 and x1.00). Measured
 # offline; the summaries are kept in profiles/.
 TRAFFIC_BYTES = {
-    "decode_chain": (36_805 + 33_024) * 1024,            # per chain launch, 16 slots x 1 row
-    "verify_chain": (167_932 + 1_585_152) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
-    "prefill_2048_rows": (141_315 + 148_482 + 152_700 + 36_864 + 65_571 + 32_768 + 172 + 144) * 1024,
-    "mark_state_pages": (69_984 + 70_788) * 1024,
+    "decode_chain": (36_794 + 33_024) * 1024,            # per plain chain launch, 16 slots x 1 row
+    "verify_chain": (167_880 + 1_585_201) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
+    "prefill_2048_rows": (148_356 + 150_175 + 152_705 + 36_865 + 65_755 + 32_912) * 1024,   # intra, inter, norm: read + written
+    "mark_state_pages": (69_930 + 70_852) * 1024,
 }
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
@@ -246,7 +246,7 @@ def bench_prefill(steps, warmup, stream, cpu=True):
         "tok_per_s_per_layer": total / (ms * 1e-3), "ms_per_8192_tokens": ms,
         "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": TRAFFIC_BYTES["prefill_2048_rows"], "traffic_unit": "B per 2048-row call (4 kernels)",
+                     "traffic": TRAFFIC_BYTES["prefill_2048_rows"], "traffic_unit": "B per 2048-row call (3 kernels)",
                      "kernel": "prefill (intra + inter + norm + conv advance, whole call)",
                      "flops_per_token": 11_709_099, "hbm_GBps_compulsory": io_bytes / (ms * 1e-3) / 1e9,
                      "hbm_frac": io_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
