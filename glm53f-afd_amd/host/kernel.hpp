@@ -362,7 +362,9 @@ class BatchMeta {
 
 /// One layer, a batch of requests (glm53f_kda_chain_batch[_bf16state]; kernel.rs:528-679). With `ckpt` set and
 /// bf16 states it is the checkpointing verify step (glm53f_kda_verify_batch_bf16state), which never writes the
-/// pool.
+/// pool. With `advance_conv` the same launch moves every request's conv window past all its rows
+/// (glm53f_kda_chain_shift_batch[_bf16state]: what conv_shift_batch with keep = rows would do next); the windows are
+/// written then and must not overlap.
 struct ChainBatch {
     const Weights* weights = nullptr;
     RowView p;
@@ -374,6 +376,7 @@ struct ChainBatch {
     RowView out;
     const Saves* saves = nullptr;
     Buf ckpt;    // bf16 [total rows][H][128][128], or empty
+    bool advance_conv = false;
 
     Error check(const BatchMeta& meta, StateType st, void** state_out_ptr) const {
         KDA_TRY(weights->check());
@@ -388,9 +391,10 @@ struct ChainBatch {
         KDA_TRY(g.check("g", 2, 0, total, 0, (int64_t)(h * DV)));
         KDA_TRY(out.check("out", 2, 0, total, 0, (int64_t)(h * DV)));
         if (total > 1 && out.stride < h * DV) return Error::invalid("out rows overlap");
-        KDA_TRY(meta.check_regions("conv", conv, 2, 0, WINDOW * channels(h), false, [](const Request& r) { return r.conv_offset; }));
+        KDA_TRY(meta.check_regions("conv", conv, 2, 0, WINDOW * channels(h), advance_conv, [](const Request& r) { return r.conv_offset; }));
         KDA_TRY(meta.check_regions("state", state, es, 0, state_len(h), true, [](const Request& r) { return r.state_offset; }));
         *state_out_ptr = nullptr;
+        if (advance_conv && ckpt.p != nullptr) return Error::invalid("a verify round's windows wait for the commit");
         if (ckpt.p != nullptr) {
             if (st != StateType::Bf16) return Error::invalid("checkpoints need bf16 states");
             if (state_out.kind != StateOut::Skip) return Error::invalid("a checkpointing verify does not write the pool");
@@ -435,6 +439,21 @@ struct ChainBatch {
                 meta.state_off(), w.a_log.ptr<float>(), w.dt_bias.ptr<float>(), w.norm_w.ptr<glm53f_bf16>(), w.eps,
                 w.lower, op, (int64_t)out.stride, ckpt.ptr<glm53f_bf16>(), ks, vs, gs, bs, s);
             return launched(code, "glm53f_kda_verify_batch_bf16state");
+        }
+        if (advance_conv) {
+            if (st == StateType::F32)
+                code = glm53f_kda_chain_shift_batch(
+                    h32, batch, meta.cu_rows(), pp, (int64_t)p.stride, b_off, ap, (int64_t)a.stride, gp, (int64_t)g.stride,
+                    conv.ptr<glm53f_bf16>(), meta.conv_off(), w.conv_w.ptr<glm53f_bf16>(), state.ptr<float>(),
+                    reinterpret_cast<float*>(so), meta.state_off(), w.a_log.ptr<float>(), w.dt_bias.ptr<float>(),
+                    w.norm_w.ptr<glm53f_bf16>(), w.eps, w.lower, op, (int64_t)out.stride, ks, vs, gs, bs, s);
+            else
+                code = glm53f_kda_chain_shift_batch_bf16state(
+                    h32, batch, meta.cu_rows(), pp, (int64_t)p.stride, b_off, ap, (int64_t)a.stride, gp, (int64_t)g.stride,
+                    conv.ptr<glm53f_bf16>(), meta.conv_off(), w.conv_w.ptr<glm53f_bf16>(), state.ptr<glm53f_bf16>(),
+                    reinterpret_cast<glm53f_bf16*>(so), meta.state_off(), w.a_log.ptr<float>(), w.dt_bias.ptr<float>(),
+                    w.norm_w.ptr<glm53f_bf16>(), w.eps, w.lower, op, (int64_t)out.stride, ks, vs, gs, bs, s);
+            return launched(code, "glm53f_kda_chain_shift_batch");
         }
         if (st == StateType::F32)
             code = glm53f_kda_chain_batch(h32, batch, meta.cu_rows(), pp, (int64_t)p.stride, b_off, ap, (int64_t)a.stride, gp,

@@ -277,6 +277,42 @@ static void gpu_tests() {
     EXPECT(std::memcmp(rep.data(), got.data() + 2 * n, n * 4) == 0);
     EXPECT(std::memcmp(pool.data(), got.data(), 2 * n * 4) == 0);
 
+    // A decode round in one launch: the chain in place with the windows advanced == the chain, then conv_shift_batch
+    {
+        DeviceBuffer d_pool_a, d_pool_b, d_conv_a, d_conv_b, d_out_b;
+        EXPECT_OK(DeviceBuffer::from_slice(enc(pool), &d_pool_a));
+        EXPECT_OK(DeviceBuffer::from_slice(enc(pool), &d_pool_b));
+        EXPECT_OK(DeviceBuffer::from_slice(enc(convs), &d_conv_a));
+        EXPECT_OK(DeviceBuffer::from_slice(enc(convs), &d_conv_b));
+        EXPECT_OK(DeviceBuffer::zeroed(rows * h * DV * 2, &d_out_b));
+        BatchMeta m2(0);
+        EXPECT_OK(BatchMeta::create(4, &m2));
+        EXPECT_OK(m2.set({{4, 2 * WINDOW * c, 2 * n}, {2, 0, 0}}, {4, 2}));
+        ChainBatch two = cb;
+        two.ckpt = Buf(); two.saves = nullptr; two.conv = d_conv_a; two.state = d_pool_a; two.state_out = StateOut::in_place();
+        EXPECT_OK(two.launch_bf16_state(m2, stream));
+        EXPECT_OK(conv_shift_batch(h, 1, m2, d_conv_a, 0, RowView(d_p, 0, ps), 0, stream));
+        ChainBatch one = two;
+        one.conv = d_conv_b; one.state = d_pool_b; one.out = RowView::dense(d_out_b, h * DV); one.advance_conv = true;
+        EXPECT_OK(one.launch_bf16_state(m2, stream));
+        EXPECT_OK(stream.synchronize());
+        std::vector<uint16_t> pa, pb, ca, cbv, oa, ob2;
+        EXPECT_OK(d_pool_a.to_vec(&pa)); EXPECT_OK(d_pool_b.to_vec(&pb));
+        EXPECT_OK(d_conv_a.to_vec(&ca)); EXPECT_OK(d_conv_b.to_vec(&cbv));
+        EXPECT_OK(d_out.to_vec(&oa)); EXPECT_OK(d_out_b.to_vec(&ob2));
+        EXPECT(pa == pb);
+        EXPECT(ca == cbv);
+        EXPECT(oa == ob2);
+        // a verify round cannot advance its windows, and shared windows are rejected
+        { ChainBatch x = one; x.ckpt = d_ck; x.state_out = StateOut::skip(); EXPECT_INVALID(x.launch_bf16_state(m2, stream)); }
+        BatchMeta m3(0);
+        EXPECT_OK(BatchMeta::create(4, &m3));
+        EXPECT_OK(m3.set({{4, 0, 2 * n}, {2, 0, 0}}, {4, 2}));
+        EXPECT_INVALID(one.launch_bf16_state(m3, stream));
+        { ChainBatch x = one; x.advance_conv = false; EXPECT_OK(x.launch_bf16_state(m3, stream)); }
+        EXPECT_OK(stream.synchronize());
+    }
+
     // Prefill through the wrapper against the literal recurrence
     PrefillWorkspace ws;
     EXPECT_OK(PrefillWorkspace::within(h, 1, 1 << 20, &ws));
