@@ -86,6 +86,21 @@ def test_prefill_64_heads_and_layouts():
         assert np.array_equal(c2, cv), kw
 
 
+def test_prefill_rows_off_the_128_bit_boundaries():
+    """Strides that are no multiple of 8 elements, and projection rows that start 6 bytes into a 16-byte piece (beta
+    logits of 3 heads in front): the kernels' 16-bit input path and the norm's 32-bit path give the dense result's
+    bits."""
+    for heads, t, kws in ((4, 150, ({"pad": 2}, {"pad": 6, "in_place": True})), (3, 70, ({"b_first": True}, {"b_first": True, "pad": 2}))):
+        p, conv, s0, rows = case(heads, t, 95 + heads)
+        out, st, cv = hs.prefill_gpu(p, conv, s0, rows)
+        check_against_oracle(p, conv, s0, rows, out, st, cv, f"{heads} heads")
+        for kw in kws:
+            o2, s2, c2 = hs.prefill_gpu(p, conv, s0, rows, **kw)
+            assert np.array_equal(hs.bits(o2), hs.bits(out)), kw
+            assert np.array_equal(hs.bits(s2), hs.bits(st)), kw
+            assert np.array_equal(c2, cv), kw
+
+
 @pytest.mark.parametrize("bf16_state", [False, True])
 def test_batched_equals_per_request_bitwise(bf16_state):
     """gpu_prefill.rs:302-373: requests of 37, 0, 100, 16 and 1 rows in shuffled slots against one launch per
