@@ -1,0 +1,231 @@
+// BF16 weight GEMV for 1 to 8 rows (gfx950): HBM-bound, every weight byte streamed once with 128-bit nontemporal
+// loads. Numerical contract: the reference's host model, crates/glm53f-forward/src/reference.rs:27-71 (kernel
+// counterpart kernels/gemv_bf16.cu:29-106 with 32-lane warps): 32 partial sums per output and K split, each an
+// fma chain over k = lo + 8 l + 256 i + j; an xor butterfly over 16, 8, 4, 2, 1; splits added in order.
+//
+// Here half a wave (32 lanes) plays the model's 32 partials of two outputs at once. The activations of the
+// workgroup's K range sit in LDS (bf16, staged once per range piece), so a lane reads them as 128-bit pieces next
+// to the weight pieces it streams; a workgroup of 8 half-waves owns 16 outputs.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "glm53f_fwd_gemv.h"
+
+namespace fwd_gemv {
+namespace {
+
+constexpr int kInvalid = 1;                       // hipErrorInvalidValue
+constexpr int THREADS = 256;
+constexpr int OUTS = 2;                           // outputs per half-wave
+constexpr int BLOCK_OUTS = (THREADS / 32) * OUTS; // 16 outputs per workgroup
+constexpr int STEP = 256;                         // values of K per step of a half-wave: 32 lanes x 8
+constexpr int UNROLL = 4;                         // steps whose weight pieces are requested together
+constexpr int LDS_BYTES = 64 * 1024;              // staged activations: rows x range piece x 2 bytes at most
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 hwbf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float lo16(uint32_t v) { return __uint_as_float(v << 16); }
+__device__ __forceinline__ float hi16(uint32_t v) { return __uint_as_float(v & 0xffff0000u); }
+__device__ __forceinline__ uint16_t f2bf(float x) { return __builtin_bit_cast(uint16_t, (__bf16)x); }
+
+// x[lane ^ M] inside a row of 16 lanes by DPP (quad permutes, a rotation by 8, two masked shifts by 4).
+template <int M>
+__device__ __forceinline__ float lane_xor16(float x) {
+    const int xi = __float_as_int(x);
+    if constexpr (M == 1) return __int_as_float(__builtin_amdgcn_update_dpp(0, xi, 0xB1, 0xf, 0xf, true));
+    if constexpr (M == 2) return __int_as_float(__builtin_amdgcn_update_dpp(0, xi, 0x4E, 0xf, 0xf, true));
+    if constexpr (M == 8) return __int_as_float(__builtin_amdgcn_update_dpp(0, xi, 0x128, 0xf, 0xf, true));
+    if constexpr (M == 4) {
+        const int lo = __builtin_amdgcn_update_dpp(0, xi, 0x104, 0xf, 0x5, false);
+        return __int_as_float(__builtin_amdgcn_update_dpp(lo, xi, 0x114, 0xf, 0xa, false));
+    }
+    return x;
+}
+
+// The model's warp_sum over the 32 lanes of a half-wave (crates/glm53f-layers/src/math.rs:76-88): every lane ends
+// with the same bits.
+__device__ __forceinline__ float half_wave_sum(float v) {
+    v = v + __shfl_xor(v, 16, 64);
+    v = v + lane_xor16<8>(v);
+    v = v + lane_xor16<4>(v);
+    v = v + lane_xor16<2>(v);
+    v = v + lane_xor16<1>(v);
+    return v;
+}
+
+template <bool F32>
+__device__ __forceinline__ void store_out(void* out, long long idx, float v) {
+    if constexpr (F32) static_cast<float*>(out)[idx] = v;
+    else static_cast<uint16_t*>(out)[idx] = f2bf(v);
+}
+
+// grid (ceil(n / 16), ksplit, groups). kp: the piece of a split's K range staged at a time (a multiple of 256,
+// rows * kp * 2 bytes of LDS).
+template <int M, bool F32>
+__global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restrict__ x, long long ldx, long long x_gs,
+                                                       const uint16_t* __restrict__ w, long long ldw, long long w_gs,
+                                                       int n, int kc, int kp, float* __restrict__ partials,
+                                                       unsigned* __restrict__ sync, void* __restrict__ out,
+                                                       long long ldo, long long o_gs) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    uint16_t* xs = reinterpret_cast<uint16_t*>(smem);                 // [M][kp]
+    const int t = threadIdx.x, hw = t >> 5, l = t & 31;
+    const int g = blockIdx.z, split = blockIdx.y, nsplit = gridDim.y;
+    const int o0 = blockIdx.x * BLOCK_OUTS + hw * OUTS;               // n % 8 == 0: o0 < n means o0 + 1 < n
+    const bool live = o0 < n;
+    const int lo = split * kc;
+    const uint16_t* xg = x + g * x_gs + lo;
+    const uint16_t* w0 = w + g * w_gs + (long long)(live ? o0 : 0) * ldw + lo;
+
+    float acc[OUTS][M];
+#pragma unroll
+    for (int r = 0; r < OUTS; ++r)
+#pragma unroll
+        for (int m = 0; m < M; ++m) acc[r][m] = 0.0f;
+
+    for (int p0 = 0; p0 < kc; p0 += kp) {
+        const int pw = min(kp, kc - p0);                              // this piece's width, a multiple of 8
+        if (p0 > 0) __syncthreads();
+        for (int e = t; e < M * (pw / 8); e += THREADS) {
+            const int m = e / (pw / 8), c = e - m * (pw / 8);
+            *reinterpret_cast<u32x4*>(xs + m * kp + 8 * c) = *reinterpret_cast<const u32x4*>(xg + m * ldx + p0 + 8 * c);
+        }
+        __syncthreads();
+        if (!live) continue;
+        // lane l takes k = p0 + 8 l + 256 i of the piece while that is inside it
+        for (int k0 = 8 * l; k0 < pw; k0 += STEP * UNROLL) {
+            u32x4 wv[UNROLL][OUTS];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+                for (int r = 0; r < OUTS; ++r)
+                    if (k0 + STEP * u < pw)
+                        wv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w0 + r * ldw + p0 + k0 + STEP * u));
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (k0 + STEP * u >= pw) break;
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    const u32x4 xv = *reinterpret_cast<const u32x4*>(xs + m * kp + k0 + STEP * u);
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const float xa = lo16(xv[d]), xb = hi16(xv[d]);
+#pragma unroll
+                        for (int r = 0; r < OUTS; ++r) {
+                            acc[r][m] = __builtin_fmaf(xa, lo16(wv[u][r][d]), acc[r][m]);
+                            acc[r][m] = __builtin_fmaf(xb, hi16(wv[u][r][d]), acc[r][m]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    void* og = F32 ? static_cast<void*>(static_cast<float*>(out) + g * o_gs)
+                   : static_cast<void*>(static_cast<uint16_t*>(out) + g * o_gs);
+    if (live) {
+#pragma unroll
+        for (int r = 0; r < OUTS; ++r)
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const float v = half_wave_sum(acc[r][m]);
+                if (l == ((r * M + m) & 31)) {
+                    if (nsplit > 1) partials[(((long long)g * nsplit + split) * M + m) * n + o0 + r] = v;
+                    else store_out<F32>(og, (long long)m * ldo + o0 + r, v);
+                }
+            }
+    }
+    if (nsplit == 1) return;
+
+    // The last workgroup of this block of outputs to finish adds the splits in split order. Counters: one per 8
+    // outputs as the caller sized them; this workgroup uses the one of its first 8.
+    __shared__ int last;
+    __threadfence();
+    __syncthreads();
+    unsigned* counter = sync + (long long)g * (n / 8) + 2 * blockIdx.x;
+    if (t == 0) last = atomicAdd(counter, 1u) == (unsigned)(nsplit - 1);
+    __syncthreads();
+    if (!last) return;
+    __threadfence();
+    if (t == 0) *counter = 0;                     // every split of this block has signalled
+    const long long split_stride = (long long)M * n;
+    for (int e = t; e < BLOCK_OUTS * M; e += THREADS) {
+        const int m = e / BLOCK_OUTS, o = blockIdx.x * BLOCK_OUTS + e % BLOCK_OUTS;
+        if (o >= n) continue;
+        const long long base = ((long long)g * nsplit * M + m) * n + o;
+        float s = __hip_atomic_load(partials + base, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int kk = 1; kk < nsplit; ++kk)
+            s = s + __hip_atomic_load(partials + base + kk * split_stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        store_out<F32>(og, (long long)m * ldo + o, s);
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <int M, bool F32>
+int32_t launch_m(const uint16_t* x, long long ldx, long long x_gs, const uint16_t* w, long long ldw, long long w_gs,
+                 int groups, int n, int k, int ksplit, float* partials, unsigned* sync, void* out, long long ldo,
+                 long long o_gs, hipStream_t stream) {
+    const int kc = k / ksplit;
+    int kp = LDS_BYTES / (2 * M) / STEP * STEP;   // the widest piece that fits, a multiple of 256
+    if (kp > kc) kp = (kc + 7) / 8 * 8;
+    const size_t lds = (size_t)M * kp * 2;        // 64 KiB at most: within the default limit of a launch
+    const dim3 grid((unsigned)((n + BLOCK_OUTS - 1) / BLOCK_OUTS), (unsigned)ksplit, (unsigned)groups);
+    gemv_kernel<M, F32><<<grid, THREADS, lds, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, kc, kp, partials, sync, out, ldo,
+                                                        o_gs);
+    return (int32_t)hipGetLastError();
+}
+
+template <bool F32>
+int32_t launch(const uint16_t* x, long long ldx, long long x_gs, const uint16_t* w, long long ldw, long long w_gs,
+               int groups, int rows, int n, int k, int ksplit, float* partials, unsigned* sync, void* out, long long ldo,
+               long long o_gs, hipStream_t stream) {
+    switch (rows) {
+        case 1: return launch_m<1, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+        case 2: return launch_m<2, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+        case 3: return launch_m<3, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+        case 4: return launch_m<4, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+        case 5: return launch_m<5, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+        case 6: return launch_m<6, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+        case 7: return launch_m<7, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+        case 8: return launch_m<8, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+        default: return kInvalid;
+    }
+}
+
+}  // namespace
+}  // namespace fwd_gemv
+
+extern "C" int32_t glm53f_fwd_gemv_ksplit(int32_t groups, int32_t n, int32_t k) {
+    if (groups < 1 || n < 8 || k < 8) return 1;
+    const long long blocks = (long long)(n / 8) * groups;
+    if (blocks >= 512) return 1;
+    int best = 1;
+    for (int d = 2; k / d >= 1024; ++d) {
+        if (k % (256 * d) != 0) continue;
+        best = d;
+        if (blocks * d >= 512) break;
+    }
+    return best;
+}
+
+// The reference's checks in the reference's order (gemv_bf16.cu:158-164).
+extern "C" int32_t glm53f_fwd_gemv_bf16(const uint16_t* x, int64_t ldx, int64_t x_gstride, const uint16_t* w,
+                                        int64_t ldw, int64_t w_gstride, int32_t groups, int32_t rows, int32_t n,
+                                        int32_t k, int32_t ksplit, float* partials, uint32_t* sync, void* out,
+                                        int32_t out_f32, int64_t ldo, int64_t o_gstride, ihipStream_t* stream) {
+    using namespace fwd_gemv;
+    if (groups < 1 || groups > 65535 || rows < 1 || rows > 8 || n < 8 || n % 8 || k < 8 || k % 8 || ksplit < 1 ||
+        ksplit > 65535 || k % ksplit || (k / ksplit) % 8)
+        return kInvalid;
+    if (!x || !w || !aligned16(x) || !aligned16(w) || !out || ldx % 8 || ldw % 8 || x_gstride % 8 || w_gstride % 8 ||
+        ldx < k || ldw < k || ldo < n)
+        return kInvalid;
+    if (ksplit > 1 && (!partials || !sync)) return kInvalid;
+    return out_f32 ? launch<true>(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, partials, sync, out,
+                                  ldo, o_gstride, stream)
+                   : launch<false>(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, partials, sync,
+                                   out, ldo, o_gstride, stream);
+}

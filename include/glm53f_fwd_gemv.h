@@ -1,0 +1,50 @@
+/* BF16 weight GEMV for MI355X (gfx950): the projections of a decode or verify step (1 to 8 rows), streamed from
+ * HBM once.
+ *
+ * Drop-in boundary: names, argument order and meaning of crates/glm53f-forward/kernels/glm53f_forward.h:19-47,
+ * bound by crates/glm53f-forward/src/ffi.rs:10-40 and called by crates/glm53f-forward/src/gemm.rs:238-291
+ * (`Gemm::gemv`; the KDA projections of forward.rs:3494-3542 reach it through `Gemm::bf16`). Only the stream handle
+ * changes: a HIP stream.
+ *
+ * Conventions (reference header :4-10): device pointers; strides in ELEMENTS; the return value is a hipError_t as
+ * int32: 0 on success, 1 (hipErrorInvalidValue) when the host rejects an argument, otherwise the launch error.
+ * Asynchronous on `stream`; nothing is allocated, freed or synchronized inside.
+ *
+ * Numerics (reference header :24-31, host model crates/glm53f-forward/src/reference.rs:27-71): for every K split,
+ * 32 partial sums per output: partial l accumulates fma(x[k], w[k], acc) over k = lo + 8 l + 256 i + j (i outer,
+ * j = 0..7); the 32 partials are added by an xor butterfly over offsets 16, 8, 4, 2, 1; the splits are added in
+ * split order; the result is stored as f32 or rounded to bf16 (nearest even). A row's result depends on that row's
+ * inputs and on (n, k, ksplit) only, never on `rows`: a verify window gives the bits of serial decode steps.
+ */
+#ifndef GLM53F_FWD_GEMV_H
+#define GLM53F_FWD_GEMV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+struct ihipStream_t;
+
+/** out[g][m][o] = sum_k x[g][m][k] * w[g][o][k] for g < groups, m < rows (1..8), o < n: x at
+ *  x + g*x_gstride + m*ldx, w row o at w + g*w_gstride + o*ldw, out at out + g*o_gstride + m*ldo (bf16, or f32
+ *  when out_f32 != 0). n % 8 == 0, k % 8 == 0, ldx, ldw, x_gstride, w_gstride % 8 == 0, x and w 16-byte aligned;
+ *  ksplit divides k and every split is a multiple of 8 wide (use glm53f_fwd_gemv_ksplit). ksplit > 1 needs
+ *  `partials` (f32 [groups][ksplit][rows][n]) and `sync` (at least groups * n / 8 zeroed counters, left zeroed).
+ *  (reference: glm53f_forward.h:21-41, gemv_bf16.cu:29-139, :154-170) */
+int32_t glm53f_fwd_gemv_bf16(const uint16_t* x, int64_t ldx, int64_t x_gstride, const uint16_t* w, int64_t ldw,
+                             int64_t w_gstride, int32_t groups, int32_t rows, int32_t n, int32_t k, int32_t ksplit,
+                             float* partials, uint32_t* sync, void* out, int32_t out_f32, int64_t ldo,
+                             int64_t o_gstride, struct ihipStream_t* stream);
+
+/** The K splits the GEMV uses for an [n][k] weight in `groups` groups: the fewest splits, each at least 1,024 wide
+ *  and a multiple of 256, that give at least 512 blocks of 8 outputs. Shape only; part of the numerical contract.
+ *  (reference: glm53f_forward.h:43-45, gemv_bf16.cu:141-152) */
+int32_t glm53f_fwd_gemv_ksplit(int32_t groups, int32_t n, int32_t k);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

@@ -1,0 +1,148 @@
+"""The BF16 GEMV through the C ABI against its model, bit for bit (after the reference's
+crates/glm53f-forward/tests/gemv.rs:97-177): the reference's five shapes (K splits, several splits, no split,
+grouped with a small K, an n that is no multiple of 16) with BF16 and f32 outputs; every row count 1..8 and a row's
+independence of the rows beside it; padded strides; a split that is no multiple of 256 wide; the argument checks of
+kernels/gemv_bf16.cu:158-164; the counters left zeroed; the KDA projection's shape (4096 -> 24,640)."""
+import numpy as np
+import pytest
+import torch
+
+from glm53f_forward import ffi as fwd
+from oracle import gemv_oracle as go
+
+import harness as hs
+
+pytestmark = pytest.mark.gpu
+DEV = hs.DEV
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+class Scratch:
+    """The engine's split-K scratch (crates/glm53f-forward/src/gemm.rs:143-171): 2^20 floats, 2^16 zeroed counters."""
+
+    def __init__(self):
+        self.partials = torch.empty(1 << 20, dtype=torch.float32, device=DEV)
+        self.sync = torch.zeros(1 << 16, dtype=torch.int32, device=DEV)
+
+
+def bf16_normal(rng, shape, sigma):
+    return go.bf16_round((rng.standard_normal(shape) * sigma).astype(np.float32))
+
+
+def run(sc, x, w, rows, ksplit, f32_out, *, ldx=None, ldw=None, ldo=None, xg=None, wg=None, og=None):
+    """x [groups][rows_total][k] bits, w [groups][n][k] bits -> f32 [groups][rows][n] (bf16 outputs widened)."""
+    groups, _, k = x.shape
+    n = w.shape[1]
+    ldx, ldw, ldo = ldx or k, ldw or k, ldo or n
+    xg = xg if xg is not None else x.shape[1] * ldx
+    wg = wg if wg is not None else n * ldw
+    og = og if og is not None else rows * ldo
+    xs = np.full(groups * xg + 8, 0x7FC0, dtype=np.uint16)           # NaN filler: a read outside the rows shows
+    ws = np.full(groups * wg + 8, 0x7FC0, dtype=np.uint16)
+    for g in range(groups):
+        for m in range(x.shape[1]):
+            xs[g * xg + m * ldx:g * xg + m * ldx + k] = x[g, m]
+        for o in range(n):
+            ws[g * wg + o * ldw:g * wg + o * ldw + k] = w[g, o]
+    d_x, d_w = dev(xs), dev(ws)
+    out = torch.full((groups * og + 8,), -7.0, dtype=torch.float32 if f32_out else torch.bfloat16, device=DEV)
+    rc = fwd.glm53f_fwd_gemv_bf16(hs.ptr(d_x), ldx, xg, hs.ptr(d_w), ldw, wg, groups, rows, n, k, ksplit,
+                                  hs.ptr(sc.partials), hs.ptr(sc.sync), hs.ptr(out), int(f32_out), ldo, og, None)
+    assert rc == 0, rc
+    hs.sync()
+    o = out.float().cpu().numpy()
+    got = np.stack([np.stack([o[g * og + m * ldo:g * og + m * ldo + n] for m in range(rows)]) for g in range(groups)])
+    gaps = np.ones(o.size, dtype=bool)
+    for g in range(groups):
+        for m in range(rows):
+            gaps[g * og + m * ldo:g * og + m * ldo + n] = False
+    assert (o[gaps] == -7.0).all()                                    # nothing written beside the outputs
+    return got
+
+
+def model(x, w, rows, ksplit, f32_out):
+    outs = []
+    for g in range(x.shape[0]):
+        v = go.gemv_bf16(x[g, :rows], w[g], ksplit)
+        outs.append(v if f32_out else go.bf16_to_f32(go.bf16_round(v)))
+    return np.stack(outs)
+
+
+SHAPES = [(1, 64, 4096, False), (1, 288, 4096, True), (1, 1024, 1536, False), (2, 512, 128, False), (1, 4096, 4096, True),
+          (1, 24, 520, True), (3, 8, 2048, False)]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"g{s[0]}-n{s[1]}-k{s[2]}-{'f32' if s[3] else 'bf16'}")
+def test_gemv_matches_its_model_and_is_row_independent(shape):
+    groups, n, k, f32_out = shape
+    sc = Scratch()
+    rng = np.random.default_rng(11 + n + k)
+    ksplit = fwd.glm53f_fwd_gemv_ksplit(groups, n, k)
+    assert ksplit == go.gemv_ksplit(groups, n, k)
+    w = bf16_normal(rng, (groups, n, k), 0.02)
+    x = bf16_normal(rng, (groups, 8, k), 1.0)
+    got = run(sc, x, w, 8, ksplit, f32_out)
+    want = model(x, w, 8, ksplit, f32_out)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), f"{(got != want).sum()} values differ"
+    for rows in range(1, 9):
+        part = run(sc, x, w, rows, ksplit, f32_out)
+        assert np.array_equal(part.view(np.uint32), got[:, :rows].view(np.uint32)), rows
+    assert int(sc.sync.abs().sum()) == 0                              # the counters are left zeroed
+
+
+def test_gemv_with_padded_strides_and_every_split_count():
+    sc = Scratch()
+    rng = np.random.default_rng(5)
+    groups, n, k = 2, 40, 2048
+    w = bf16_normal(rng, (groups, n, k), 0.02)
+    x = bf16_normal(rng, (groups, 5, k), 1.0)
+    for ksplit in (1, 2, 4, 8):
+        for f32_out in (False, True):
+            got = run(sc, x, w, 5, ksplit, f32_out, ldx=k + 8, ldw=k + 16, ldo=n + 3, xg=5 * (k + 8) + 64,
+                      wg=n * (k + 16) + 8, og=5 * (n + 3) + 1)
+            want = model(x, w, 5, ksplit, f32_out)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (ksplit, f32_out)
+    assert int(sc.sync.abs().sum()) == 0
+
+
+def test_gemv_kda_projection_shape():
+    """The KDA input projection of a decode step: 4096 -> 24,640 (q | k | v and the beta logits), one row and eight."""
+    sc = Scratch()
+    rng = np.random.default_rng(6)
+    n, k = 24_640, 4096
+    w = bf16_normal(rng, (1, n, k), 0.02)
+    x = bf16_normal(rng, (1, 8, k), 1.0)
+    assert fwd.glm53f_fwd_gemv_ksplit(1, n, k) == 1
+    got8 = run(sc, x, w, 8, 1, False)
+    got1 = run(sc, x, w, 1, 1, False)
+    assert np.array_equal(got1.view(np.uint32), got8[:, :1].view(np.uint32))
+    sample = rng.permutation(n)[:2048]
+    want = model(x, w[:, sample], 8, 1, False)
+    assert np.array_equal(got8[:, :, sample].view(np.uint32), want.view(np.uint32))
+
+
+def test_gemv_argument_checks():
+    sc = Scratch()
+    buf = torch.zeros(1 << 16, dtype=torch.bfloat16, device=DEV)
+    out = torch.zeros(1 << 12, dtype=torch.float32, device=DEV)
+    x, w, o, pa, sy = hs.ptr(buf), hs.ptr(buf, 8192), hs.ptr(out), hs.ptr(sc.partials), hs.ptr(sc.sync)
+
+    def call(**kw):
+        a = dict(x=x, ldx=256, xg=0, w=w, ldw=256, wg=0, groups=1, rows=2, n=16, k=256, ksplit=1, pa=pa, sy=sy, o=o,
+                 f32=1, ldo=16, og=0)
+        a.update(kw)
+        return fwd.glm53f_fwd_gemv_bf16(a["x"], a["ldx"], a["xg"], a["w"], a["ldw"], a["wg"], a["groups"], a["rows"],
+                                        a["n"], a["k"], a["ksplit"], a["pa"], a["sy"], a["o"], a["f32"], a["ldo"],
+                                        a["og"], None)
+
+    assert call() == 0
+    for bad in (dict(groups=0), dict(groups=70000), dict(rows=0), dict(rows=9), dict(n=0), dict(n=12), dict(k=4),
+                dict(k=260), dict(ksplit=0), dict(ksplit=3), dict(k=2064, ldx=2064, ldw=2064, ksplit=4),
+                dict(x=x + 2), dict(w=w + 6), dict(o=None), dict(ldx=260), dict(ldw=257), dict(xg=4), dict(wg=12),
+                dict(ldx=248), dict(ldw=128), dict(ldo=8), dict(k=2048, ldx=2048, ldw=2048, ksplit=2, pa=None),
+                dict(k=2048, ldx=2048, ldw=2048, ksplit=2, sy=None), dict(x=None), dict(w=None)):
+        assert call(**bad) == 1, bad
+    hs.sync()

@@ -135,7 +135,7 @@ def declarations():
 
 def test_library_exports_the_declared_row_entry_points():
     decl = declarations()
-    assert set(decl) == set(rows_ffi.PROTOTYPES) == {"glm53f_fwd_gather_rows", "glm53f_fwd_scatter_rows"}
+    assert set(decl) == {"glm53f_fwd_gather_rows", "glm53f_fwd_scatter_rows"} <= set(rows_ffi.PROTOTYPES)
     lib = rows_ffi.lib()
     for name, nargs in decl.items():
         assert hasattr(lib, name), name
