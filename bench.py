@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the KDA hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|mark|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|mark|gemv|copy]
 
 Prints ONE JSON line. The headline `value` is the decode step's state traffic in GB/s in the 16-slot decode configuration
 (16 slots x 1 token out of a 48-slot bf16 pool, 64 heads, 34 layers each with its own pool so the working set
@@ -431,6 +431,59 @@ def bench_mark(steps, warmup, stream, cpu=True):
     return res
 
 
+# ------------------------------------------------------------------------------------------------ gemv
+
+def bench_gemv(steps, warmup, stream, cpu=True):
+    """The BF16 projections next to the KDA core in a decode or verify step (crates/glm53f-forward/src/forward.rs:
+    3494-3542, :3772-3789): the input projection 4096 -> 24,640 with 1 and 8 rows, and the output projection
+    8192 -> 4096. Weights streamed from HBM once per call; four copies of each weight in turn, so that no call finds
+    its weight in the 256 MB Infinity Cache."""
+    from glm53f_forward import ffi as fwd
+    gen = torch.Generator(device=DEV).manual_seed(8)
+    partials = torch.empty(1 << 20, dtype=torch.float32, device=DEV)
+    sync = torch.zeros(1 << 16, dtype=torch.int32, device=DEV)
+    res = {"config": {"workload": "BF16 GEMV, weights [n][k] streamed once: kda_proj 4096 -> 24,640 (1 and 8 rows), "
+                                  "o_proj 8192 -> 4096 (1 row); four weight copies in turn"}}
+    copies = 4
+    for name, n, k, rows in (("kda_proj_1row", 24_640, 4096, 1), ("kda_proj_8rows", 24_640, 4096, 8),
+                             ("o_proj_1row", 4096, 8192, 1)):
+        w = (torch.randn(copies, n, k, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
+        x = torch.randn(8, k, device=DEV, generator=gen).to(torch.bfloat16)
+        out = torch.zeros(8, n, dtype=torch.bfloat16, device=DEV)
+        ksplit = fwd.glm53f_fwd_gemv_ksplit(1, n, k)
+        calls = [(ptr(x), k, 0, ptr(w[c]), k, 0, 1, rows, n, k, ksplit, ptr(partials), ptr(sync), ptr(out), 0, n, 0,
+                  stream.cuda_stream) for c in range(copies)]
+        turn = [0]
+
+        def one():
+            turn[0] += 1
+            check(fwd.glm53f_fwd_gemv_bf16(*calls[turn[0] % copies]), "gemv")
+
+        ms = timed(one, steps, warmup, stream)
+        wbytes = n * k * 2
+        res[name] = {"us": ms * 1e3, "weight_GBps": wbytes / (ms * 1e-3) / 1e9, "ksplit": ksplit,
+                     "frac_of_hbm_peak": wbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+        del w
+    r = res["kda_proj_1row"]
+    res["roofline"] = {"bound": "hbm", "kernel": "gemv_kernel<1, bf16 out>", "achieved": r["weight_GBps"],
+                       "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": r["frac_of_hbm_peak"],
+                       "traffic": TRAFFIC_BYTES.get("gemv_kda_proj_1row"), "algorithmic_bytes": 24_640 * 4096 * 2}
+    if cpu:
+        from oracle import gemv_oracle as go
+        rng = np.random.default_rng(2)
+        n_s, k = 512, 4096
+        wh = go.bf16_round((rng.standard_normal((n_s, k)) * 0.02).astype(np.float32))
+        xh = go.bf16_round(rng.standard_normal((1, k)).astype(np.float32))
+        reps, t0 = 0, time.perf_counter()
+        while reps < 2 or time.perf_counter() - t0 < 2.0:
+            go.gemv_bf16(xh, wh, 1)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": n_s * k * 2 / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"{reps} runs of the numpy model on 512 of the 24,640 outputs, one row"}
+    return res
+
+
 # ------------------------------------------------------------------------------------------------ main
 
 # ------------------------------------------------------------------------------------------------ copy
@@ -450,7 +503,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "copy"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "gemv", "copy"], default=None)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -498,6 +551,12 @@ def main():
         if args.only == "mark":
             line.update({"value": mk["roofline"]["achieved"], "ms_per_step": mk["scatter_state_pages_ms"],
                          "roofline": mk["roofline"], "config": mk["config"]})
+    if args.only in (None, "gemv"):
+        gv = bench_gemv(args.steps, args.warmup, stream, cpu=not args.no_cpu)
+        line["gemv"] = gv
+        if args.only == "gemv":
+            line.update({"value": gv["roofline"]["achieved"], "ms_per_step": gv["kda_proj_1row"]["us"] / 1e3,
+                         "roofline": gv["roofline"], "config": gv["config"]})
     if args.only == "copy":
         cp = bench_copy(args.steps, args.warmup, stream)
         line.update({"copy": cp, "value": cp["GBps"], "ms_per_step": cp["ms"],

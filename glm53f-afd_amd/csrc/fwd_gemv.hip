@@ -3,9 +3,10 @@
 // counterpart kernels/gemv_bf16.cu:29-106 with 32-lane warps): 32 partial sums per output and K split, each an
 // fma chain over k = lo + 8 l + 256 i + j; an xor butterfly over 16, 8, 4, 2, 1; splits added in order.
 //
-// Here half a wave (32 lanes) plays the model's 32 partials of two outputs at once. The activations of the
-// workgroup's K range sit in LDS (bf16, staged once per range piece), so a lane reads them as 128-bit pieces next
-// to the weight pieces it streams; a workgroup of 8 half-waves owns 16 outputs.
+// Here half a wave (32 lanes) plays the model's 32 partials of OUTS outputs at once (1 or 2: more outputs share
+// the activations a lane reads, fewer give more workgroups for a small n). The activations of the workgroup's K
+// range sit in LDS as f32 (widened once when they are staged), so a lane reads them as 128-bit pieces next to the
+// weight pieces it streams; a workgroup of 8 half-waves owns 8 OUTS outputs.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -16,15 +17,12 @@ namespace {
 
 constexpr int kInvalid = 1;                       // hipErrorInvalidValue
 constexpr int THREADS = 256;
-constexpr int OUTS = 2;                           // outputs per half-wave
-constexpr int BLOCK_OUTS = (THREADS / 32) * OUTS; // 16 outputs per workgroup
 constexpr int STEP = 256;                         // values of K per step of a half-wave: 32 lanes x 8
-constexpr int UNROLL = 4;                         // steps whose weight pieces are requested together
-constexpr int LDS_BYTES = 64 * 1024;              // staged activations: rows x range piece x 2 bytes at most
+constexpr int LDS_BYTES = 64 * 1024;              // staged activations: rows x range piece x 4 bytes at most
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 hwbf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float lo16(uint32_t v) { return __uint_as_float(v << 16); }
 __device__ __forceinline__ float hi16(uint32_t v) { return __uint_as_float(v & 0xffff0000u); }
@@ -61,19 +59,21 @@ __device__ __forceinline__ void store_out(void* out, long long idx, float v) {
     else static_cast<uint16_t*>(out)[idx] = f2bf(v);
 }
 
-// grid (ceil(n / 16), ksplit, groups). kp: the piece of a split's K range staged at a time (a multiple of 256,
-// rows * kp * 2 bytes of LDS).
-template <int M, bool F32>
+// grid (ceil(n / (8 OUTS)), ksplit, groups). kp: the piece of a split's K range staged at a time (a multiple of
+// 256, rows * kp * 4 bytes of LDS). UNROLL: steps whose weight pieces are requested together.
+template <int M, int OUTS, bool F32>
 __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restrict__ x, long long ldx, long long x_gs,
                                                        const uint16_t* __restrict__ w, long long ldw, long long w_gs,
                                                        int n, int kc, int kp, float* __restrict__ partials,
                                                        unsigned* __restrict__ sync, void* __restrict__ out,
                                                        long long ldo, long long o_gs) {
+    constexpr int BLOCK_OUTS = (THREADS / 32) * OUTS;
+    constexpr int UNROLL = OUTS == 1 ? 8 : 4;
     extern __shared__ __align__(16) unsigned char smem[];
-    uint16_t* xs = reinterpret_cast<uint16_t*>(smem);                 // [M][kp]
+    float* xs = reinterpret_cast<float*>(smem);                       // [M][kp]
     const int t = threadIdx.x, hw = t >> 5, l = t & 31;
     const int g = blockIdx.z, split = blockIdx.y, nsplit = gridDim.y;
-    const int o0 = blockIdx.x * BLOCK_OUTS + hw * OUTS;               // n % 8 == 0: o0 < n means o0 + 1 < n
+    const int o0 = blockIdx.x * BLOCK_OUTS + hw * OUTS;               // n % 8 == 0: o0 < n means o0 + OUTS <= n
     const bool live = o0 < n;
     const int lo = split * kc;
     const uint16_t* xg = x + g * x_gs + lo;
@@ -87,39 +87,63 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
 
     for (int p0 = 0; p0 < kc; p0 += kp) {
         const int pw = min(kp, kc - p0);                              // this piece's width, a multiple of 8
-        if (p0 > 0) __syncthreads();
-        for (int e = t; e < M * (pw / 8); e += THREADS) {
-            const int m = e / (pw / 8), c = e - m * (pw / 8);
-            *reinterpret_cast<u32x4*>(xs + m * kp + 8 * c) = *reinterpret_cast<const u32x4*>(xg + m * ldx + p0 + 8 * c);
-        }
-        __syncthreads();
-        if (!live) continue;
-        // lane l takes k = p0 + 8 l + 256 i of the piece while that is inside it
-        for (int k0 = 8 * l; k0 < pw; k0 += STEP * UNROLL) {
-            u32x4 wv[UNROLL][OUTS];
+        // lane l takes k = p0 + 8 l + 256 i of the piece while that is inside it. The weight pieces of UNROLL steps
+        // are requested together, the next set before the current one is worked on, the first before the
+        // activations are staged.
+        auto request = [&](u32x4 (&wv)[UNROLL][OUTS], int k0) {
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-                for (int r = 0; r < OUTS; ++r)
-                    if (k0 + STEP * u < pw)
-                        wv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w0 + r * ldw + p0 + k0 + STEP * u));
+                for (int r = 0; r < OUTS; ++r)   // unconditional (a step past the piece re-reads its last one)
+                    wv[u][r] = __builtin_nontemporal_load(
+                        reinterpret_cast<const u32x4*>(w0 + r * ldw + p0 + min(k0 + STEP * u, pw - 8)));
+        };
+        auto work = [&](const u32x4 (&wv)[UNROLL][OUTS], int k0) {
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 if (k0 + STEP * u >= pw) break;
+                float wf[OUTS][8];
 #pragma unroll
-                for (int m = 0; m < M; ++m) {
-                    const u32x4 xv = *reinterpret_cast<const u32x4*>(xs + m * kp + k0 + STEP * u);
+                for (int r = 0; r < OUTS; ++r)
 #pragma unroll
                     for (int d = 0; d < 4; ++d) {
-                        const float xa = lo16(xv[d]), xb = hi16(xv[d]);
+                        wf[r][2 * d] = lo16(wv[u][r][d]);
+                        wf[r][2 * d + 1] = hi16(wv[u][r][d]);
+                    }
 #pragma unroll
-                        for (int r = 0; r < OUTS; ++r) {
-                            acc[r][m] = __builtin_fmaf(xa, lo16(wv[u][r][d]), acc[r][m]);
-                            acc[r][m] = __builtin_fmaf(xb, hi16(wv[u][r][d]), acc[r][m]);
-                        }
+                for (int m = 0; m < M; ++m) {
+                    const f32x4* xp = reinterpret_cast<const f32x4*>(xs + m * kp + k0 + STEP * u);
+                    const f32x4 xa = xp[0], xb = xp[1];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float xv = j < 4 ? xa[j] : xb[j - 4];
+#pragma unroll
+                        for (int r = 0; r < OUTS; ++r) acc[r][m] = __builtin_fmaf(xv, wf[r][j], acc[r][m]);
                     }
                 }
             }
+        };
+        u32x4 wa[UNROLL][OUTS], wb[UNROLL][OUTS];
+        int k0 = 8 * l;
+        request(wa, k0);
+        if (p0 > 0) __syncthreads();
+        for (int e = t; e < M * (pw / 8); e += THREADS) {
+            const int m = e / (pw / 8), c = e - m * (pw / 8);
+            const u32x4 v = *reinterpret_cast<const u32x4*>(xg + m * ldx + p0 + 8 * c);
+            f32x4* dst = reinterpret_cast<f32x4*>(xs + m * kp + 8 * c);
+            dst[0] = f32x4{lo16(v[0]), hi16(v[0]), lo16(v[1]), hi16(v[1])};
+            dst[1] = f32x4{lo16(v[2]), hi16(v[2]), lo16(v[3]), hi16(v[3])};
+        }
+        __syncthreads();
+        if (!live) continue;
+        while (k0 < pw) {                         // in pairs, so that the two register sets are compile-time choices
+            request(wb, k0 + STEP * UNROLL);
+            work(wa, k0);
+            k0 += STEP * UNROLL;
+            if (k0 >= pw) break;
+            request(wa, k0 + STEP * UNROLL);
+            work(wb, k0);
+            k0 += STEP * UNROLL;
         }
     }
 
@@ -144,7 +168,7 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
     __shared__ int last;
     __threadfence();
     __syncthreads();
-    unsigned* counter = sync + (long long)g * (n / 8) + 2 * blockIdx.x;
+    unsigned* counter = sync + (long long)g * (n / 8) + OUTS * blockIdx.x;
     if (t == 0) last = atomicAdd(counter, 1u) == (unsigned)(nsplit - 1);
     __syncthreads();
     if (!last) return;
@@ -164,18 +188,33 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+template <int M, int OUTS, bool F32>
+int32_t launch_mo(const uint16_t* x, long long ldx, long long x_gs, const uint16_t* w, long long ldw, long long w_gs,
+                  int groups, int n, int k, int ksplit, float* partials, unsigned* sync, void* out, long long ldo,
+                  long long o_gs, hipStream_t stream) {
+    const int kc = k / ksplit;
+    // the widest piece of the K range whose activations fit 32 KiB (64 KiB for one row: no second piece up to
+    // k = 16,384), a multiple of 256: more workgroups per CU matter more than fewer barriers
+    int kp = (M == 1 ? LDS_BYTES : LDS_BYTES / 2) / (4 * M) / STEP * STEP;
+    if (kp > kc) kp = kc;
+    const size_t lds = (size_t)M * kp * 4;
+    const int block_outs = (THREADS / 32) * OUTS;
+    const dim3 grid((unsigned)((n + block_outs - 1) / block_outs), (unsigned)ksplit, (unsigned)groups);
+    gemv_kernel<M, OUTS, F32><<<grid, THREADS, lds, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, kc, kp, partials, sync,
+                                                              out, ldo, o_gs);
+    return (int32_t)hipGetLastError();
+}
+
+// Outputs per half-wave: two when that still leaves the chip four workgroups per CU (they share the activations a
+// lane reads), else one. (Four measured slower: 250 registers, two waves per SIMD.)
 template <int M, bool F32>
 int32_t launch_m(const uint16_t* x, long long ldx, long long x_gs, const uint16_t* w, long long ldw, long long w_gs,
                  int groups, int n, int k, int ksplit, float* partials, unsigned* sync, void* out, long long ldo,
                  long long o_gs, hipStream_t stream) {
-    const int kc = k / ksplit;
-    int kp = LDS_BYTES / (2 * M) / STEP * STEP;   // the widest piece that fits, a multiple of 256
-    if (kp > kc) kp = (kc + 7) / 8 * 8;
-    const size_t lds = (size_t)M * kp * 2;        // 64 KiB at most: within the default limit of a launch
-    const dim3 grid((unsigned)((n + BLOCK_OUTS - 1) / BLOCK_OUTS), (unsigned)ksplit, (unsigned)groups);
-    gemv_kernel<M, F32><<<grid, THREADS, lds, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, kc, kp, partials, sync, out, ldo,
-                                                        o_gs);
-    return (int32_t)hipGetLastError();
+    const long long blocks8 = (long long)(n / 8) * ksplit * groups;   // workgroups with one output per half-wave
+    if (n % 16 == 0 && blocks8 >= 2 * 1024)
+        return launch_mo<M, 2, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+    return launch_mo<M, 1, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
 }
 
 template <bool F32>
