@@ -38,6 +38,7 @@ TRAFFIC_BYTES = {
     "verify_chain": (167_880 + 1_585_201) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
     "prefill_2048_rows": (148_356 + 150_175 + 152_705 + 36_865 + 65_755 + 32_912) * 1024,   # intra, inter, norm: read + written
     "mark_state_pages": (69_930 + 70_852) * 1024,
+    "gemv_kda_proj_1row": (197_885 + 48) * 1024,         # per launch: the weights once, the activations, the outputs
 }
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
@@ -442,11 +443,12 @@ def bench_gemv(steps, warmup, stream, cpu=True):
     gen = torch.Generator(device=DEV).manual_seed(8)
     partials = torch.empty(1 << 20, dtype=torch.float32, device=DEV)
     sync = torch.zeros(1 << 16, dtype=torch.int32, device=DEV)
-    res = {"config": {"workload": "BF16 GEMV, weights [n][k] streamed once: kda_proj 4096 -> 24,640 (1 and 8 rows), "
-                                  "o_proj 8192 -> 4096 (1 row); four weight copies in turn"}}
+    res = {"config": {"workload": "BF16 GEMV, weights [n][k] streamed once: kda_proj 4096 -> 24,640 and o_proj "
+                                  "8192 -> 4096 with 1 to 8 rows; four weight copies in turn"}}
     copies = 4
-    for name, n, k, rows in (("kda_proj_1row", 24_640, 4096, 1), ("kda_proj_8rows", 24_640, 4096, 8),
-                             ("o_proj_1row", 4096, 8192, 1)):
+    for name, n, k, rows in (("kda_proj_1row", 24_640, 4096, 1), ("kda_proj_4rows", 24_640, 4096, 4),
+                             ("kda_proj_8rows", 24_640, 4096, 8), ("o_proj_1row", 4096, 8192, 1),
+                             ("o_proj_8rows", 4096, 8192, 8)):
         w = (torch.randn(copies, n, k, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
         x = torch.randn(8, k, device=DEV, generator=gen).to(torch.bfloat16)
         out = torch.zeros(8, n, dtype=torch.bfloat16, device=DEV)
@@ -464,6 +466,17 @@ def bench_gemv(steps, warmup, stream, cpu=True):
         res[name] = {"us": ms * 1e3, "weight_GBps": wbytes / (ms * 1e-3) / 1e9, "ksplit": ksplit,
                      "frac_of_hbm_peak": wbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
         del w
+    # the same projections over a 2048-row prefill segment: the vendor GEMM (hipBLASLt through torch.matmul), which the
+    # reference's engine takes above 8 rows (cuBLAS there); reported, not built here
+    for name, n, k in (("kda_proj_2048rows_vendor_gemm", 24_640, 4096), ("o_proj_2048rows_vendor_gemm", 4096, 8192)):
+        w = (torch.randn(n, k, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
+        xr = torch.randn(2048, k, device=DEV, generator=gen).to(torch.bfloat16)
+        o2 = torch.empty(2048, n, dtype=torch.bfloat16, device=DEV)
+        ms = timed(lambda: torch.matmul(xr, w.t(), out=o2), max(2, steps // 4), 2, stream)
+        flops = 2.0 * 2048 * n * k
+        res[name] = {"us": ms * 1e3, "TFLOPs": flops / (ms * 1e-3) / 1e12,
+                     "frac_of_mfma_peak": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+        del w, xr, o2
     r = res["kda_proj_1row"]
     res["roofline"] = {"bound": "hbm", "kernel": "gemv_kernel<1, bf16 out>", "achieved": r["weight_GBps"],
                        "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": r["frac_of_hbm_peak"],

@@ -186,6 +186,126 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
     }
 }
 
+// The same contract for three rows and more, where a lane's arithmetic (rows x 8 fused multiply-adds per weight
+// word pair) and its reads of the activations weigh as much as the weight stream: half a wave owns eight outputs
+// and walks the K steps in the outer loop, so that the rows' activations of a step are read from LDS once for all
+// eight (each accumulator still sees its products in the order of the model). 128 lanes per workgroup, 32 outputs;
+// taken when that still gives two workgroups per CU (64-lane workgroups for a smaller n measured slower than the
+// kernel above).
+constexpr int WIDE_THREADS = 128, WIDE_OUTS = 8;
+
+template <int M, bool F32>
+__global__ void __launch_bounds__(WIDE_THREADS) gemv_wide_kernel(const uint16_t* __restrict__ x, long long ldx,
+                                                                 long long x_gs, const uint16_t* __restrict__ w,
+                                                                 long long ldw, long long w_gs, int n, int kc, int kp,
+                                                                 float* __restrict__ partials,
+                                                                 unsigned* __restrict__ sync, void* __restrict__ out,
+                                                                 long long ldo, long long o_gs) {
+    constexpr int BLOCK_OUTS = (WIDE_THREADS / 32) * WIDE_OUTS;
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* xs = reinterpret_cast<float*>(smem);                       // [M][kp]
+    const int t = threadIdx.x, hw = t >> 5, l = t & 31;
+    const int g = blockIdx.z, split = blockIdx.y, nsplit = gridDim.y;
+    const int o0 = blockIdx.x * BLOCK_OUTS + hw * WIDE_OUTS;
+    const bool live = o0 < n;
+    const int lo = split * kc;
+    const uint16_t* xg = x + g * x_gs + lo;
+    const uint16_t* w0 = w + g * w_gs + (long long)(live ? o0 : 0) * ldw + lo;
+
+    float acc[WIDE_OUTS][M];
+#pragma unroll
+    for (int r = 0; r < WIDE_OUTS; ++r)
+#pragma unroll
+        for (int m = 0; m < M; ++m) acc[r][m] = 0.0f;
+
+    for (int p0 = 0; p0 < kc; p0 += kp) {
+        const int pw = min(kp, kc - p0);
+        auto request = [&](u32x4 (&wv)[WIDE_OUTS], int k0) {         // unconditional, as above
+#pragma unroll
+            for (int r = 0; r < WIDE_OUTS; ++r)
+                wv[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w0 + r * ldw + p0 + min(k0, pw - 8)));
+        };
+        auto work = [&](const u32x4 (&wv)[WIDE_OUTS], int k0) {
+            float xr[M][8];
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const f32x4* xp = reinterpret_cast<const f32x4*>(xs + m * kp + k0);
+                const f32x4 xa = xp[0], xb = xp[1];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { xr[m][j] = xa[j]; xr[m][4 + j] = xb[j]; }
+            }
+#pragma unroll
+            for (int r = 0; r < WIDE_OUTS; ++r) {
+                float wf[8];
+#pragma unroll
+                for (int d = 0; d < 4; ++d) { wf[2 * d] = lo16(wv[r][d]); wf[2 * d + 1] = hi16(wv[r][d]); }
+#pragma unroll
+                for (int m = 0; m < M; ++m)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[r][m] = __builtin_fmaf(xr[m][j], wf[j], acc[r][m]);
+            }
+        };
+        u32x4 wa[WIDE_OUTS], wb[WIDE_OUTS];
+        int k0 = 8 * l;
+        request(wa, k0);
+        if (p0 > 0) __syncthreads();
+        for (int e = t; e < M * (pw / 8); e += WIDE_THREADS) {
+            const int m = e / (pw / 8), c = e - m * (pw / 8);
+            const u32x4 v = *reinterpret_cast<const u32x4*>(xg + m * ldx + p0 + 8 * c);
+            f32x4* dst = reinterpret_cast<f32x4*>(xs + m * kp + 8 * c);
+            dst[0] = f32x4{lo16(v[0]), hi16(v[0]), lo16(v[1]), hi16(v[1])};
+            dst[1] = f32x4{lo16(v[2]), hi16(v[2]), lo16(v[3]), hi16(v[3])};
+        }
+        __syncthreads();
+        if (!live) continue;
+        while (k0 < pw) {
+            request(wb, k0 + STEP);
+            work(wa, k0);
+            k0 += STEP;
+            if (k0 >= pw) break;
+            request(wa, k0 + STEP);
+            work(wb, k0);
+            k0 += STEP;
+        }
+    }
+
+    void* og = F32 ? static_cast<void*>(static_cast<float*>(out) + g * o_gs)
+                   : static_cast<void*>(static_cast<uint16_t*>(out) + g * o_gs);
+    if (live) {
+#pragma unroll
+        for (int r = 0; r < WIDE_OUTS; ++r)
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const float v = half_wave_sum(acc[r][m]);
+                if (l == ((r * M + m) & 31)) {
+                    if (nsplit > 1) partials[(((long long)g * nsplit + split) * M + m) * n + o0 + r] = v;
+                    else store_out<F32>(og, (long long)m * ldo + o0 + r, v);
+                }
+            }
+    }
+    if (nsplit == 1) return;
+
+    __shared__ int last;                          // as above: the last workgroup of these outputs adds the splits
+    __threadfence();
+    __syncthreads();
+    unsigned* counter = sync + (long long)g * (n / 8) + (BLOCK_OUTS / 8) * blockIdx.x;
+    if (t == 0) last = atomicAdd(counter, 1u) == (unsigned)(nsplit - 1);
+    __syncthreads();
+    if (!last) return;
+    __threadfence();
+    if (t == 0) *counter = 0;
+    const long long split_stride = (long long)M * n;
+    for (int e = t; e < BLOCK_OUTS * M; e += WIDE_THREADS) {
+        const int m = e / BLOCK_OUTS, o = blockIdx.x * BLOCK_OUTS + e % BLOCK_OUTS;
+        if (o >= n) continue;
+        const long long base = ((long long)g * nsplit * M + m) * n + o;
+        float s = __hip_atomic_load(partials + base, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int kk = 1; kk < nsplit; ++kk)
+            s = s + __hip_atomic_load(partials + base + kk * split_stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        store_out<F32>(og, (long long)m * ldo + o, s);
+    }
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <int M, int OUTS, bool F32>
@@ -212,6 +332,15 @@ int32_t launch_m(const uint16_t* x, long long ldx, long long x_gs, const uint16_
                  int groups, int n, int k, int ksplit, float* partials, unsigned* sync, void* out, long long ldo,
                  long long o_gs, hipStream_t stream) {
     const long long blocks8 = (long long)(n / 8) * ksplit * groups;   // workgroups with one output per half-wave
+    if (M >= 3 && blocks8 >= 4 * 512) {                                // 32 outputs per workgroup: two per CU and more
+        const int kc = k / ksplit;
+        int kp = LDS_BYTES / 2 / (4 * M) / STEP * STEP;
+        if (kp > kc) kp = kc;
+        const dim3 grid((unsigned)((n + 31) / 32), (unsigned)ksplit, (unsigned)groups);
+        gemv_wide_kernel<M, F32><<<grid, WIDE_THREADS, (size_t)M * kp * 4, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, kc, kp,
+                                                                                     partials, sync, out, ldo, o_gs);
+        return (int32_t)hipGetLastError();
+    }
     if (n % 16 == 0 && blocks8 >= 2 * 1024)
         return launch_mo<M, 2, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
     return launch_mo<M, 1, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from glm53f_forward import ffi as fwd
+from glm53f_forward.gemm import Bf16Mat, Gemm, GemmError, GemmPolicy
 from oracle import gemv_oracle as go
 
 import harness as hs
@@ -106,6 +107,14 @@ def test_gemv_with_padded_strides_and_every_split_count():
             want = model(x, w, 5, ksplit, f32_out)
             assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (ksplit, f32_out)
     assert int(sc.sync.abs().sum()) == 0
+    # enough outputs for the eight-outputs-per-half-wave kernel, with K splits (the rule itself would not split here)
+    n = 8200
+    w = bf16_normal(rng, (1, n, 1024), 0.02)
+    x = bf16_normal(rng, (1, 4, 1024), 1.0)
+    for ksplit in (1, 2):
+        got = run(sc, x, w, 4, ksplit, True, ldo=n + 8)
+        assert np.array_equal(got.view(np.uint32), model(x, w, 4, ksplit, True).view(np.uint32)), ksplit
+    assert int(sc.sync.abs().sum()) == 0
 
 
 def test_gemv_kda_projection_shape():
@@ -146,3 +155,41 @@ def test_gemv_argument_checks():
                 dict(k=2048, ldx=2048, ldw=2048, ksplit=2, sy=None), dict(x=None), dict(w=None)):
         assert call(**bad) == 1, bad
     hs.sync()
+
+
+def test_engine_dispatch_and_the_vendor_gemm_within_rounding():
+    """crates/glm53f-forward/tests/gemv.rs:179-254: the GEMV through the engine wrapper, the vendor GEMM for more rows
+    than the policy gives the GEMV, and their agreement within f32 rounding (relative RMS < 1e-5)."""
+    rng = np.random.default_rng(12)
+    n, k = 2048, 4096
+    w = dev(bf16_normal(rng, (n, k), 0.02)).view(torch.bfloat16)
+    x = dev(bf16_normal(rng, (16, k), 1.0)).view(torch.bfloat16)
+    gemm = Gemm()
+    mat = Bf16Mat.of(w)
+    assert mat.bytes() == n * k * 2 and Gemm.gemv_ksplit(mat) == 2
+
+    def run_f32(rows, blas):
+        out = torch.zeros(rows, n, dtype=torch.float32, device=DEV)
+        (gemm.blas if blas else gemm.gemv)(x.data_ptr(), k, 0, mat, rows, out.data_ptr(), n, 0, True)
+        hs.sync()
+        return out.cpu().numpy()
+
+    g8, b8 = run_f32(8, False), run_f32(8, True)
+    rel = np.sqrt(np.mean((g8 - b8) ** 2) / np.mean(g8 ** 2))
+    assert rel < 1e-5, rel
+    want = go.gemv_bf16(x[:8].view(torch.int16).cpu().numpy().view(np.uint16), w.view(torch.int16).cpu().numpy().view(np.uint16), 2)
+    assert np.array_equal(g8.view(np.uint32), want.view(np.uint32))
+    # the policy: 8 rows and fewer take the GEMV (the model's bits), more the vendor GEMM (bf16 of a close value)
+    out = torch.zeros(16, n, dtype=torch.bfloat16, device=DEV)
+    gemm.bf16(x.data_ptr(), k, 0, mat, 8, out.data_ptr(), n, 0, False)
+    hs.sync()
+    got8 = out[:8].float().cpu().numpy()
+    assert np.array_equal(got8, go.bf16_to_f32(go.bf16_round(want)))
+    gemm.bf16(x.data_ptr(), k, 0, mat, 16, out.data_ptr(), n, 0, False)
+    hs.sync()
+    got16 = out.float().cpu().numpy()
+    assert np.max(np.abs(got16[:8] - got8)) <= np.max(np.abs(got8)) * 2.0 ** -7
+    with pytest.raises(GemmError):
+        Gemm(GemmPolicy(gemv_max_rows=9))
+    with pytest.raises(GemmError):                                    # the launcher's own checks surface as errors
+        gemm.gemv(x.data_ptr() + 2, k, 0, mat, 8, out.data_ptr(), n, 0, False)
