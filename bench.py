@@ -248,7 +248,7 @@ def bench_prefill(steps, warmup, stream, cpu=True):
         "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": TRAFFIC_BYTES["prefill_2048_rows"], "traffic_unit": "B per 2048-row call (3 kernels)",
-                     "kernel": "prefill (intra + inter + norm + conv advance, whole call)",
+                     "kernel": "prefill (intra + inter + norm with the conv window advance, whole call)",
                      "flops_per_token": 11_709_099, "hbm_GBps_compulsory": io_bytes / (ms * 1e-3) / 1e9,
                      "hbm_frac": io_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
         "config": {"workload": "benchmark configuration 2: T=8192 as 4 calls of 2048 rows on one slot, H=64, chunk 64, "
