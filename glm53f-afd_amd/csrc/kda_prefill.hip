@@ -605,21 +605,29 @@ __device__ __forceinline__ void store_state_elem4(bf16_t* p, const f32x4 v) {
     *reinterpret_cast<uint2*>(p) = make_uint2(f2bf2(v[0], v[1]), f2bf2(v[2], v[3]));
 }
 
-// One chunk's operands of inter_kernel as a wave holds them: MFMA fragments straight from the workspace. Wave w
-// owns rows 16 w .. 16 w + 15 of the chunk (W, Qg, M, U) and keys 32 w .. 32 w + 31 of the state (Kg, e^{G_last}),
-// and nothing it loads is used by another wave, so none of it passes through LDS.
-struct InterOperands {
-    u32x4 w[4], q[4];                             // rows 16 w + l % 16, keys 32 ks + 8 (l / 16) ..
-    u32x4 m[2];                                   // rows 16 w + l % 16, chunk rows 32 ks + 8 (l / 16) ..
+// One chunk's operands of inter_kernel as a wave holds them: MFMA fragments straight from the workspace. The
+// workgroup has two kinds of wave. State wave w (waves 0..3) owns rows 16 w .. 16 w + 15 of the chunk for V' (W, U)
+// and keys 32 w .. 32 w + 31 of the state (Kg, e^{G_last}); read-out wave w (waves 4..7) owns rows 16 w .. 16 w + 15
+// of the chunk for Y (Qg, M). Nothing a wave loads is used by another wave, so none of it passes through LDS.
+struct StateOperands {
+    u32x4 w[4];                                   // rows 16 w + l % 16, keys 32 ks + 8 (l / 16) ..
     u32x4 k[2][2];                                // keys 32 w + 16 mt + l % 16, chunk rows 32 ks + 8 (l / 16) ..
-    uint2 u[NT];                                   // value 16 nt + l % 16, rows 16 w + 4 (l / 16) ..
+    uint2 u[NT];                                  // value 16 nt + l % 16, rows 16 w + 4 (l / 16) ..
     f32x4 e[2];                                   // keys 32 w + 16 mt + 4 (l / 16) ..
 };
+struct ReadoutOperands {
+    u32x4 q[4];                                   // rows 16 w + l % 16, keys 32 ks + 8 (l / 16) ..
+    u32x4 m[2];                                   // rows 16 w + l % 16, chunk rows 32 ks + 8 (l / 16) ..
+};
+constexpr int INTER_THREADS = 512;
 
 // Pass 2: one head's NV value columns of one request through the chunks of the pass, in order. The state
-// S[128 keys][NV] lives in MFMA accumulators: wave w owns keys 32 w .. 32 w + 31.
+// S[128 keys][NV] lives in the MFMA accumulators of the state waves: wave w owns keys 32 w .. 32 w + 31. Only
+// V' = U - W S and S <- e S + Kg^T V' are on the path from one chunk's state to the next; the read-out
+// Y = Qg S + M V' hangs off it, so it runs in four waves of its own beside the state waves (one of each per SIMD)
+// and the chain from chunk to chunk is two short products and two barriers.
 template <typename S>
-__global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 2))) inter_kernel(
+__global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) inter_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
         const S* state_in, S* state_out, const long long* __restrict__ state_off,
         bf16_t* __restrict__ out, long long out_stride, const unsigned char* __restrict__ ws) {
@@ -629,7 +637,10 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
     // they run on one XCD and share its L2 instead of fetching the workspace once per block.
     const int h = blockIdx.x % H, vb = blockIdx.x / H, b = blockIdx.y;
     const RowRange rr = request_rows(cu_rows, b, rows1);
-    const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave8 = __builtin_amdgcn_readfirstlane(t >> 6);
+    const bool state_wave = wave8 < 4;
+    const int wave = wave8 & 3;
     const int left = rr.rows - sub0;                              // rows of this request from this pass on
     const int nch = left <= 0 ? 0 : min(chunks, (left + CH - 1) / CH);
     if (nch == 0 && sub0 > 0) return;                             // nothing left: the state is already written
@@ -638,167 +649,191 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1,
 
     uint16_t* Sl = reinterpret_cast<uint16_t*>(smem + N_S);
     uint16_t* Vl = reinterpret_cast<uint16_t*>(smem + N_V);
-
-    // the state: accS[mt][nt][r] = S[key 32 w + 16 mt + rl + r][value NV vb + 16 nt + cl]
-    f32x4 accS[2][NT];
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            float v4[4];
-            load_state_elem4<S>(state_in + sbase + (long long)(NV * vb + SUB * nt + cl) * DK + 32 * wave + SUB * mt + rl, v4);
-            accS[mt][nt] = f32x4{v4[0], v4[1], v4[2], v4[3]};
-        }
-
     const unsigned char* wsh = ws + ((long long)b * H + h) * chunks * (long long)WS_BYTES;
     // Per-lane byte offsets of the fragments inside a chunk's workspace.
     const unsigned off_a = (unsigned)(((SUB * wave + cl) * 32 + 8 * (lane >> 4)) * 2);   // W, Qg, M: + 4096 ks
-    const unsigned off_k = (unsigned)(WS_KGT + ((32 * wave + cl) * 32 + 8 * (lane >> 4)) * 2);  // + 1024 mt + 8192 ks
-    const unsigned off_u = (unsigned)(WS_UT + ((NV * vb + cl) * CH + SUB * wave + rl) * 2);     // + 2048 nt
-    const unsigned off_e = (unsigned)(WS_E + (32 * wave + rl) * 4);                             // + 64 mt
-    // The loads of chunk C_ into operand set X_, one group at a time (each group is requested as soon as the
-    // chunk two before it has used those registers). Unconditional: past the end they repeat the last chunk.
-#define KDA_LOAD_W(X_, C_)                                                                                          \
-    {                                                                                                               \
-        const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                               \
-        _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                            \
-            X_.w[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_W + off_a + 4096 * ks);                              \
-        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                            \
-            X_.u[nt] = *reinterpret_cast<const uint2*>(src_ + off_u + 2048 * nt);                                    \
-    }
-#define KDA_LOAD_QM(X_, C_)                                                                                         \
-    {                                                                                                               \
-        const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                               \
-        _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                            \
-            X_.q[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_QG + off_a + 4096 * ks);                             \
-        _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                            \
-            X_.m[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_M + off_a + 4096 * ks);                              \
-    }
-#define KDA_LOAD_KE(X_, C_)                                                                                         \
-    {                                                                                                               \
-        const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                               \
-        _Pragma("unroll") for (int mt = 0; mt < 2; ++mt) {                                                          \
-            _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                        \
-                X_.k[mt][ks] = *reinterpret_cast<const u32x4*>(src_ + off_k + 1024 * mt + 8192 * ks);                \
-            X_.e[mt] = *reinterpret_cast<const f32x4*>(src_ + off_e + 64 * mt);                                      \
-        }                                                                                                           \
-    }
-    // S^T (fp16) for the products of a chunk
-    auto put_state = [&]() {
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto as_u4 = [](const u32x4 v) { return make_uint4(v[0], v[1], v[2], v[3]); };
+    // Both kinds of wave pass the same two barriers per chunk: after the first the state of the chunk is in LDS
+    // (and every wave is done with the V' of the chunk before), after the second its V' is.
+
+    if (state_wave) {
+        // the state: accS[mt][nt][r] = S[key 32 w + 16 mt + rl + r][value NV vb + 16 nt + cl]
+        f32x4 accS[2][NT];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const uint32_t s0 = (uint32_t)f2h(accS[mt][nt][0]) | ((uint32_t)f2h(accS[mt][nt][1]) << 16);
-                const uint32_t s1 = (uint32_t)f2h(accS[mt][nt][2]) | ((uint32_t)f2h(accS[mt][nt][3]) << 16);
-                *reinterpret_cast<uint2*>(Sl + (SUB * nt + cl) * LD128 + 32 * wave + SUB * mt + rl) = make_uint2(s0, s1);
+                float v4[4];
+                load_state_elem4<S>(state_in + sbase + (long long)(NV * vb + SUB * nt + cl) * DK + 32 * wave + SUB * mt + rl, v4);
+                accS[mt][nt] = f32x4{v4[0], v4[1], v4[2], v4[3]};
             }
-    };
-    auto as_u4 = [](const u32x4 v) { return make_uint4(v[0], v[1], v[2], v[3]); };
-
-    // Chunk c with the operands in x; each group of x is then requested again for chunk c + 2.
-    auto chunk_step = [&](const int c, InterOperands& x) __attribute__((always_inline)) {
-        const int nrows = min(CH, left - c * CH);
-        const int c2 = min(c + 2, nch - 1);
-        put_state();
-        __syncthreads();      // the state is in LDS; every wave is done with the V' of the chunk before
-        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-        // V' = U - W S: wave w takes rows 16 w .. 16 w + 15
-        uint4 sfrag[NT][4];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) sfrag[nt][ks] = frag(Sl, LD128, SUB * nt, 32 * ks, lane);
-        f32x4 accV[NT];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) accV[nt] = zero;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) accV[nt] = mfma_f16(as_u4(x.w[ks]), sfrag[nt][ks], accV[nt]);
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const uint2 u = x.u[nt];
-            const float v0 = h2f((uint16_t)(u.x & 0xffffu)) - accV[nt][0], v1 = h2f((uint16_t)(u.x >> 16)) - accV[nt][1];
-            const float v2 = h2f((uint16_t)(u.y & 0xffffu)) - accV[nt][2], v3 = h2f((uint16_t)(u.y >> 16)) - accV[nt][3];
-            const uint32_t p0 = (uint32_t)f2h(v0) | ((uint32_t)f2h(v1) << 16);
-            const uint32_t p1 = (uint32_t)f2h(v2) | ((uint32_t)f2h(v3) << 16);
-            *reinterpret_cast<uint2*>(Vl + (SUB * nt + cl) * LD64 + SUB * wave + rl) = make_uint2(p0, p1);
+        const unsigned off_k = (unsigned)(WS_KGT + ((32 * wave + cl) * 32 + 8 * (lane >> 4)) * 2);  // + 1024 mt + 8192 ks
+        const unsigned off_u = (unsigned)(WS_UT + ((NV * vb + cl) * CH + SUB * wave + rl) * 2);     // + 2048 nt
+        const unsigned off_e = (unsigned)(WS_E + (32 * wave + rl) * 4);                             // + 64 mt
+        // The loads of chunk C_ into operand set X_, one group at a time (each group is requested as soon as the
+        // chunk two before it has used those registers). Unconditional: past the end they repeat the last chunk.
+#define KDA_LOAD_W(X_, C_)                                                                                          \
+        {                                                                                                           \
+            const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
+            _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                        \
+                X_.w[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_W + off_a + 4096 * ks);                          \
+            _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                        \
+                X_.u[nt] = *reinterpret_cast<const uint2*>(src_ + off_u + 2048 * nt);                                \
         }
-        KDA_LOAD_W(x, c2)
-        __syncthreads();
-        // Y = Qg S + M V'
-        uint4 vfrag[NT][2];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) vfrag[nt][ks] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
-        f32x4 accY[NT];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) accY[nt] = zero;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) accY[nt] = mfma_f16(as_u4(x.q[ks]), sfrag[nt][ks], accY[nt]);
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) accY[nt] = mfma_f16(as_u4(x.m[ks]), vfrag[nt][ks], accY[nt]);
-        KDA_LOAD_QM(x, c2)
-        {
-            const long long grow0 = rr.row0 + sub0 + c * CH;
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int row = SUB * wave + rl + r;
-                    if (row < nrows)
-                        (out + (grow0 + row) * out_stride + h * DV + NV * vb + SUB * nt)[(unsigned)cl] = f2bf(accY[nt][r]);
-                }
+#define KDA_LOAD_KE(X_, C_)                                                                                         \
+        {                                                                                                           \
+            const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
+            _Pragma("unroll") for (int mt = 0; mt < 2; ++mt) {                                                      \
+                _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                    \
+                    X_.k[mt][ks] = *reinterpret_cast<const u32x4*>(src_ + off_k + 1024 * mt + 8192 * ks);            \
+                X_.e[mt] = *reinterpret_cast<const f32x4*>(src_ + off_e + 64 * mt);                                  \
+            }                                                                                                       \
         }
-        // S <- e^{G_last} S + Kg^T V'
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) accS[mt][nt][r] *= x.e[mt][r];
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) accS[mt][nt] = mfma_f16(as_u4(x.k[mt][ks]), vfrag[nt][ks], accS[mt][nt]);
-        }
-        KDA_LOAD_KE(x, c2)
-        if constexpr (sizeof(S) == 2) {
-            // a bf16 state is rounded at the end of every chunk, so the result does not depend on where passes end
+        // Chunk c with the operands in x; each group of x is then requested again for chunk c + 2.
+        auto chunk_step = [&](const int c, StateOperands& x) __attribute__((always_inline)) {
+            const int c2 = min(c + 2, nch - 1);
+            // S^T (fp16) for the products of the chunk
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const uint32_t s0 = (uint32_t)f2h(accS[mt][nt][0]) | ((uint32_t)f2h(accS[mt][nt][1]) << 16);
+                    const uint32_t s1 = (uint32_t)f2h(accS[mt][nt][2]) | ((uint32_t)f2h(accS[mt][nt][3]) << 16);
+                    *reinterpret_cast<uint2*>(Sl + (SUB * nt + cl) * LD128 + 32 * wave + SUB * mt + rl) = make_uint2(s0, s1);
+                }
+            __syncthreads();
+            // V' = U - W S: wave w takes rows 16 w .. 16 w + 15
+            f32x4 accV[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) accV[nt] = zero;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    accV[nt] = mfma_f16(as_u4(x.w[ks]), frag(Sl, LD128, SUB * nt, 32 * ks, lane), accV[nt]);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const uint2 u = x.u[nt];
+                const float v0 = h2f((uint16_t)(u.x & 0xffffu)) - accV[nt][0], v1 = h2f((uint16_t)(u.x >> 16)) - accV[nt][1];
+                const float v2 = h2f((uint16_t)(u.y & 0xffffu)) - accV[nt][2], v3 = h2f((uint16_t)(u.y >> 16)) - accV[nt][3];
+                const uint32_t p0 = (uint32_t)f2h(v0) | ((uint32_t)f2h(v1) << 16);
+                const uint32_t p1 = (uint32_t)f2h(v2) | ((uint32_t)f2h(v3) << 16);
+                *reinterpret_cast<uint2*>(Vl + (SUB * nt + cl) * LD64 + SUB * wave + rl) = make_uint2(p0, p1);
+            }
+            KDA_LOAD_W(x, c2)
+            __syncthreads();
+            // S <- e^{G_last} S + Kg^T V'
+            uint4 vfrag[NT][2];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) vfrag[nt][ks] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) accS[mt][nt][r] = bfround(accS[mt][nt][r]);
-        }
-    };
-    if (nch > 0) {
-        InterOperands xa, xb;                     // even and odd chunks
-        KDA_LOAD_W(xa, 0) KDA_LOAD_QM(xa, 0) KDA_LOAD_KE(xa, 0)
-        const int c1 = min(1, nch - 1);
-        KDA_LOAD_W(xb, c1) KDA_LOAD_QM(xb, c1) KDA_LOAD_KE(xb, c1)
-        // in pairs, so that the operand sets are compile-time choices; an odd last chunk follows
-        int c = 0;
+                    for (int r = 0; r < 4; ++r) accS[mt][nt][r] *= x.e[mt][r];
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) accS[mt][nt] = mfma_f16(as_u4(x.k[mt][ks]), vfrag[nt][ks], accS[mt][nt]);
+            }
+            KDA_LOAD_KE(x, c2)
+            if constexpr (sizeof(S) == 2) {
+                // a bf16 state is rounded at the end of every chunk, so the result does not depend on where passes end
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) accS[mt][nt][r] = bfround(accS[mt][nt][r]);
+            }
+        };
+        if (nch > 0) {
+            StateOperands xa, xb;                 // even and odd chunks
+            KDA_LOAD_W(xa, 0) KDA_LOAD_KE(xa, 0)
+            const int c1 = min(1, nch - 1);
+            KDA_LOAD_W(xb, c1) KDA_LOAD_KE(xb, c1)
+            // in pairs, so that the operand sets are compile-time choices; an odd last chunk follows
+            int c = 0;
 #pragma unroll 1
-        for (; c + 1 < nch; c += 2) {
-            chunk_step(c, xa);
-            chunk_step(c + 1, xb);
+            for (; c + 1 < nch; c += 2) {
+                chunk_step(c, xa);
+                chunk_step(c + 1, xb);
+            }
+            if (c < nch) chunk_step(c, xa);
         }
-        if (c < nch) chunk_step(c, xa);
+#undef KDA_LOAD_W
+#undef KDA_LOAD_KE
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                store_state_elem4(state_out + sbase + (long long)(NV * vb + SUB * nt + cl) * DK + 32 * wave + SUB * mt + rl,
+                                  accS[mt][nt]);
+    } else {
+        // rows of `out` that start on 8-byte boundaries take four values per store
+        const bool wide_out = ((reinterpret_cast<size_t>(out) | (size_t)(out_stride * 2)) & 7) == 0;
+#define KDA_LOAD_QM(X_, C_)                                                                                         \
+        {                                                                                                           \
+            const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
+            _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                        \
+                X_.q[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_QG + off_a + 4096 * ks);                         \
+            _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                        \
+                X_.m[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_M + off_a + 4096 * ks);                          \
+        }
+        auto chunk_step = [&](const int c, ReadoutOperands& x) __attribute__((always_inline)) {
+            const int nrows = min(CH, left - c * CH);
+            const int c2 = min(c + 2, nch - 1);
+            __syncthreads();
+            // Y^T = S^T Qg^T + V'^T M^T: the state and V' on the row side of the tiles, so that a lane ends up with
+            // four consecutive values of one row and stores them as one 8-byte piece
+            f32x4 accY[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) accY[nt] = zero;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    accY[nt] = mfma_f16(frag(Sl, LD128, SUB * nt, 32 * ks, lane), as_u4(x.q[ks]), accY[nt]);
+            __syncthreads();
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    accY[nt] = mfma_f16(frag(Vl, LD64, SUB * nt, 32 * ks, lane), as_u4(x.m[ks]), accY[nt]);
+            KDA_LOAD_QM(x, c2)
+            if (SUB * wave + cl < nrows) {
+                // accY[nt][r] = y[row 16 w + cl][value NV vb + 16 nt + rl + r]
+                bf16_t* orow = out + (rr.row0 + sub0 + c * CH + SUB * wave + cl) * out_stride + h * DV + NV * vb + rl;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const uint2 y4 = make_uint2(f2bf2(accY[nt][0], accY[nt][1]), f2bf2(accY[nt][2], accY[nt][3]));
+                    if (wide_out) *reinterpret_cast<uint2*>(orow + SUB * nt) = y4;
+                    else {
+                        orow[SUB * nt] = (bf16_t)(y4.x & 0xffffu); orow[SUB * nt + 1] = (bf16_t)(y4.x >> 16);
+                        orow[SUB * nt + 2] = (bf16_t)(y4.y & 0xffffu); orow[SUB * nt + 3] = (bf16_t)(y4.y >> 16);
+                    }
+                }
+            }
+        };
+        if (nch > 0) {
+            ReadoutOperands xa, xb;
+            KDA_LOAD_QM(xa, 0)
+            const int c1 = min(1, nch - 1);
+            KDA_LOAD_QM(xb, c1)
+            int c = 0;
+#pragma unroll 1
+            for (; c + 1 < nch; c += 2) {
+                chunk_step(c, xa);
+                chunk_step(c + 1, xb);
+            }
+            if (c < nch) chunk_step(c, xa);
+        }
+#undef KDA_LOAD_QM
     }
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-            store_state_elem4(state_out + sbase + (long long)(NV * vb + SUB * nt + cl) * DK + 32 * wave + SUB * mt + rl,
-                              accS[mt][nt]);
 }
 
 // The call's last launch: the conv windows' advance, and the gated RMSNorm over the bf16 read-outs the inter pass
@@ -960,7 +995,7 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
             if (rc != 0) return rc;
         }
         const S* s_in = sub0 == 0 ? state_in : state_out;
-        inter_kernel<S><<<dim3(heads * VBLOCKS, batch), THREADS, INTER_LDS, st>>>(
+        inter_kernel<S><<<dim3(heads * VBLOCKS, batch), INTER_THREADS, INTER_LDS, st>>>(
             heads, cu_rows, rows1, sub0, (int)chunks, s_in, state_out, soff, bfp(out), out_stride, ws);
         const int rc = (int)hipGetLastError();
         if (rc != 0) return rc;
