@@ -112,6 +112,11 @@ template <int N>
 __device__ __forceinline__ uint32_t row_shl_u(uint32_t x) {
     return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x100 + N, 0xf, 0xf, true);
 }
+// The value n lanes below where there is one; the other lanes (the first n of the row) keep `keep`.
+template <int N>
+__device__ __forceinline__ uint32_t row_shr_keep(uint32_t keep, uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)keep, (int)x, 0x110 + N, 0xf, 0xf, false);
+}
 template <int N>
 __device__ __forceinline__ float row_lane(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x150 + N, 0xf, 0xf, true));
@@ -121,6 +126,13 @@ __device__ __forceinline__ float row_lane(float x) {
 typedef __bf16 hwbf16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(hwbf16x2, a), __builtin_bit_cast(hwbf16x2, b), c, false);
+}
+
+// The same without an addend, in the three-operand encoding: a sum that starts here needs no zeroed accumulator.
+__device__ __forceinline__ float dot2_bf16_first(uint32_t a, uint32_t b) {
+    float r;
+    asm("v_dot2_f32_bf16 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(b));
+    return r;
 }
 
 // Eight consecutive bf16 from p. With VEC p is 16-byte aligned.
@@ -256,27 +268,27 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             const int seg = it >> 2, p = it & 3;
 #pragma unroll
             for (int d = 0; d < 4; ++d) {         // a 32-bit word holds two channels
-                // taps 0..2 are the rows above: the own rows of the lanes below, or (lanes 0..2) halo rows; where one
-                // has nothing (a shifted-in zero, a zero halo) the other has the row
+                // taps 0..2 are the rows above: the own rows of the lanes below; the first lanes of the row, which
+                // have no such lane, keep the halo row that belongs there (lane j's halo is row 16 w - 3 + j)
                 const uint32_t x3 = own[it][d], hl = halo[it][d];
-                const uint32_t x0 = row_shr_u<3>(x3) | hl;
-                const uint32_t x1 = row_shr_u<2>(x3) | row_shl_u<1>(hl);
-                const uint32_t x2 = row_shr_u<1>(x3) | row_shl_u<2>(hl);
+                const uint32_t x1 = row_shr_keep<2>(row_shl_u<1>(hl), x3);
+                const uint32_t x2 = row_shr_keep<1>(row_shl_u<2>(hl), x3);
+                const uint32_t x0 = row_shr_keep<3>(hl, x3);
                 float s2[2];
 #pragma unroll
                 for (int k = 0; k < 2; ++k) {
                     const u32x4 w = cw_s[seg * DK + 32 * g + 8 * p + 2 * d + k];
-                    float acc = dot2_bf16(x0, w[0], 0.0f);
+                    float acc = dot2_bf16_first(x0, w[0]);
                     acc = dot2_bf16(x1, w[1], acc);
                     acc = dot2_bf16(x2, w[2], acc);
                     acc = dot2_bf16(x3, w[3], acc);
                     s2[k] = acc * fast_sigmoid(acc);
                 }
                 const uint32_t pair = f2bf2(s2[0], s2[1]);        // the one bf16 rounding
-                const float r0f = __uint_as_float(pair << 16), r1f = __uint_as_float(pair & 0xffff0000u);
-                if (seg == 0) { qr[4 * p + d] = pair; ssq = __builtin_fmaf(r0f, r0f, ssq); ssq = __builtin_fmaf(r1f, r1f, ssq); }
-                if (seg == 1) { kr[4 * p + d] = pair; ssk = __builtin_fmaf(r0f, r0f, ssk); ssk = __builtin_fmaf(r1f, r1f, ssk); }
+                if (seg == 0) { qr[4 * p + d] = pair; ssq = dot2_bf16(pair, pair, ssq); }
+                if (seg == 1) { kr[4 * p + d] = pair; ssk = dot2_bf16(pair, pair, ssk); }
                 if (seg == 2) {
+                    const float r0f = __uint_as_float(pair << 16), r1f = __uint_as_float(pair & 0xffff0000u);
                     VT[(32 * g + 8 * p + 2 * d) * LD64 + R] = f2h(r0f);
                     VT[(32 * g + 8 * p + 2 * d + 1) * LD64 + R] = f2h(r1f);
                 }
