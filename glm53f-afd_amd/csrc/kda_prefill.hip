@@ -160,9 +160,11 @@ __device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
 
 // Pass 1: the chunks of one head of one request, everything that does not need the state, into their workspace
 // slots. Wave w owns sub-chunk w of a chunk (rows 16 w .. 16 w + 15); in the elementwise phases lane l holds row
-// l % 16 and the 32 channels 32 (l / 16) .. + 31 of it. That is the operand layout of the matrix cores for
-// products that contract over channels, so the tiles of L and M take their row side straight from registers (the
-// diagonal ones both sides); what contracts over rows later (k e^G, v, Kg) is written transposed, 16 bits at a time.
+// l % 16 and 32 channels of it: with g = l / 16, the four pieces of eight channels 32 p + 8 g .. + 7, p = 0..3 (the
+// four lanes of a row then read 64 consecutive bytes with every load, and write 64 with every store of Qg). That
+// is the operand layout of the matrix cores for products that contract over channels, so the tiles of L and M take
+// their row side straight from registers (the diagonal ones both sides); what contracts over rows later (k e^G, v,
+// Kg) is written transposed, 16 bits at a time.
 template <bool VEC>
 __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) intra_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
@@ -213,9 +215,9 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     u32x4 own[12];
     auto load_own = [&](int first_row) {
         const int rel = min(first_row + (int)(t & 15) + SUB * (int)(t >> 6), rr.rows - 1);
-        const bf16_t* src = P + (rr.row0 + rel) * p_stride + h * DK + 32 * ((t >> 4) & 3);
+        const bf16_t* src = P + (rr.row0 + rel) * p_stride + h * DK + 8 * ((t >> 4) & 3);
 #pragma unroll
-        for (int it = 0; it < 12; ++it) own[it] = load8<VEC>(src + (long long)(it >> 2) * H * DK + 8 * (it & 3));
+        for (int it = 0; it < 12; ++it) own[it] = load8<VEC>(src + (long long)(it >> 2) * H * DK + 32 * (it & 3));
     };
     load_own(sub0 + c_first * CH);
 #pragma unroll 1
@@ -224,7 +226,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // otherwise the per-lane addresses of the body are hoisted out of the chunk loop and spill.
     asm volatile("" : "+v"(t));
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63;
-    const int i = lane & 15, g = lane >> 4;       // this lane's row of the sub-chunk and its group of 32 channels
+    const int i = lane & 15, g = lane >> 4;       // this lane's row of the sub-chunk and its set of 32 channels
     const int r0 = sub0 + c * CH;                 // the chunk's first row inside the request
     const int n = min(CH, rr.rows - r0);          // its real rows
     if (n <= 0) break;
@@ -234,11 +236,11 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // row and counts as g = 0)
     u32x4 av[4];
     {
-        const bf16_t* arow = A + (rr.row0 + r0 + min(R, n - 1)) * a_stride + h * DK + 32 * g;
+        const bf16_t* arow = A + (rr.row0 + r0 + min(R, n - 1)) * a_stride + h * DK + 8 * g;
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            if constexpr (VEC) av[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(arow + 8 * p));
-            else av[p] = load8<false>(arow + 8 * p);
+            if constexpr (VEC) av[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(arow + 32 * p));
+            else av[p] = load8<false>(arow + 32 * p);
         }
     }
 
@@ -258,9 +260,9 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             if (i < WINDOW) {
                 const int hrel = min(r0 + SUB * wave - WINDOW + i, rr.rows - 1);
                 const bf16_t* hsrc = (hrel < 0 ? cs + (long long)(hrel + WINDOW) * C : P + (rr.row0 + hrel) * p_stride) +
-                                     h * DK + 32 * g;
+                                     h * DK + 8 * g;
 #pragma unroll
-                for (int it = 0; it < 12; ++it) halo[it] = load8<VEC>(hsrc + (long long)(it >> 2) * H * DK + 8 * (it & 3));
+                for (int it = 0; it < 12; ++it) halo[it] = load8<VEC>(hsrc + (long long)(it >> 2) * H * DK + 32 * (it & 3));
             }
         }
 #pragma unroll
@@ -277,7 +279,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 float s2[2];
 #pragma unroll
                 for (int k = 0; k < 2; ++k) {
-                    const u32x4 w = cw_s[seg * DK + 32 * g + 8 * p + 2 * d + k];
+                    const u32x4 w = cw_s[seg * DK + 32 * p + 8 * g + 2 * d + k];
                     float acc = dot2_bf16_first(x0, w[0]);
                     acc = dot2_bf16(x1, w[1], acc);
                     acc = dot2_bf16(x2, w[2], acc);
@@ -289,8 +291,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 if (seg == 1) { kr[4 * p + d] = pair; ssk = dot2_bf16(pair, pair, ssk); }
                 if (seg == 2) {
                     const float r0f = __uint_as_float(pair << 16), r1f = __uint_as_float(pair & 0xffff0000u);
-                    VT[(32 * g + 8 * p + 2 * d) * LD64 + R] = f2h(r0f);
-                    VT[(32 * g + 8 * p + 2 * d + 1) * LD64 + R] = f2h(r1f);
+                    VT[(32 * p + 8 * g + 2 * d) * LD64 + R] = f2h(r0f);
+                    VT[(32 * p + 8 * g + 2 * d + 1) * LD64 + R] = f2h(r1f);
                 }
             }
         }
@@ -308,8 +310,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         const uint32_t keep = R < n ? 0xffffffffu : 0u;    // a row past the end counts as g = 0
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            const f32x4 d0 = *reinterpret_cast<const f32x4*>(dtb_s + 32 * g + 8 * p);
-            const f32x4 d1 = *reinterpret_cast<const f32x4*>(dtb_s + 32 * g + 8 * p + 4);
+            const f32x4 d0 = *reinterpret_cast<const f32x4*>(dtb_s + 32 * p + 8 * g);
+            const f32x4 d1 = *reinterpret_cast<const f32x4*>(dtb_s + 32 * p + 8 * g + 4);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float dtb = e < 4 ? d0[e] : d1[e - 4];
@@ -325,7 +327,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         if (i == SUB - 1) {
 #pragma unroll
             for (int p = 0; p < 8; ++p)
-                *reinterpret_cast<f32x4*>(tot + wave * DK + 32 * g + 4 * p) = f32x4{G[4 * p], G[4 * p + 1], G[4 * p + 2], G[4 * p + 3]};
+                *reinterpret_cast<f32x4*>(tot + wave * DK + 32 * (p >> 1) + 8 * g + 4 * (p & 1)) = f32x4{G[4 * p], G[4 * p + 1], G[4 * p + 2], G[4 * p + 3]};
         }
     }
     if (t < CH) {
@@ -393,12 +395,12 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     {
         f32x4 accL = zero, accM = zero;
         uint16_t* kgT = reinterpret_cast<uint16_t*>(wsc + WS_KGT);
-        const float* eB = fac + wave * DK + 32 * g;
-        const float* eSuf = fac + (4 + wave) * DK + 32 * g;
+        const float* eB = fac + wave * DK + 8 * g;
+        const float* eSuf = fac + (4 + wave) * DK + 8 * g;
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            const f32x4 b0 = *reinterpret_cast<const f32x4*>(eB + 8 * p), b1 = *reinterpret_cast<const f32x4*>(eB + 8 * p + 4);
-            const f32x4 s0 = *reinterpret_cast<const f32x4*>(eSuf + 8 * p), s1 = *reinterpret_cast<const f32x4*>(eSuf + 8 * p + 4);
+            const f32x4 b0 = *reinterpret_cast<const f32x4*>(eB + 32 * p), b1 = *reinterpret_cast<const f32x4*>(eB + 32 * p + 4);
+            const f32x4 s0 = *reinterpret_cast<const f32x4*>(eSuf + 32 * p), s1 = *reinterpret_cast<const f32x4*>(eSuf + 32 * p + 4);
             float qg[8], kc[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -418,15 +420,15 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 ke1[ch] = kh * e1;
                 qe1[ch] = qh * e1;
                 const float fb = e < 4 ? b0[e] : b1[e - 4], fs = e < 4 ? s0[e] : s1[e - 4];
-                keT[(32 * g + ch) * LD64 + R] = f2h(ke1[ch] * fb);
-                kgT[panel_index(DK, 32 * g + ch, R)] = f2h(kh * col2 * fs);
+                keT[(32 * p + 8 * g + e) * LD64 + R] = f2h(ke1[ch] * fb);
+                kgT[panel_index(DK, 32 * p + 8 * g + e, R)] = f2h(kh * col2 * fs);
                 qg[e] = qe1[ch] * fb;
                 kc[e] = kh * col2;
             }
-            *reinterpret_cast<u32x4*>(wsc + WS_QG + panel_index(CH, R, 32 * g + 8 * p) * 2) =
+            *reinterpret_cast<u32x4*>(wsc + WS_QG + panel_index(CH, R, 32 * p + 8 * g) * 2) =
                 u32x4{pack_h2(qg[0], qg[1]), pack_h2(qg[2], qg[3]), pack_h2(qg[4], qg[5]), pack_h2(qg[6], qg[7])};
             if (wave < 3)
-                *reinterpret_cast<u32x4*>(KcE + (wave * SUB + i) * LD128 + 32 * g + 8 * p) =
+                *reinterpret_cast<u32x4*>(KcE + (wave * SUB + i) * LD128 + 32 * p + 8 * g) =
                     u32x4{pack_h2(kc[0], kc[1]), pack_h2(kc[2], kc[3]), pack_h2(kc[4], kc[5]), pack_h2(kc[6], kc[7])};
         }
         put_L(accL, wave, wave);
@@ -434,17 +436,17 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     }
     __syncthreads();                              // the column operands of every sub-chunk are in place
     // tiles left of the diagonal: rows of sub-chunk `wave` against the columns of sub-chunk cb. In MFMA step s lane
-    // group g supplies channels 32 g + 8 s .. + 7 on both sides (which k a lane supplies is free as long as both
+    // group g supplies channels 32 s + 8 g .. + 7 on both sides (which k a lane supplies is free as long as both
     // operands agree).
 #pragma unroll 1
     for (int cb = 0; cb < wave; ++cb) {
-        const float* df = fac + factor_index(wave, cb) * DK + 32 * g;
-        const uint16_t* kcol = KcE + (cb * SUB + i) * LD128 + 32 * g;
+        const float* df = fac + factor_index(wave, cb) * DK + 8 * g;
+        const uint16_t* kcol = KcE + (cb * SUB + i) * LD128 + 8 * g;
         f32x4 accL = zero, accM = zero;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const f32x4 d0 = *reinterpret_cast<const f32x4*>(df + 8 * s), d1 = *reinterpret_cast<const f32x4*>(df + 8 * s + 4);
-            const uint4 bcol = *reinterpret_cast<const uint4*>(kcol + 8 * s);
+            const f32x4 d0 = *reinterpret_cast<const f32x4*>(df + 32 * s), d1 = *reinterpret_cast<const f32x4*>(df + 32 * s + 4);
+            const uint4 bcol = *reinterpret_cast<const uint4*>(kcol + 32 * s);
             float ak[8], aq[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -591,8 +593,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
 }
 
 // LDS map of inter_kernel, bytes: only what the waves share.
-constexpr int N_S = 0;                            // fp16 [NV][LD128]: the state, transposed
-constexpr int N_V = N_S + NV * LD128 * 2;         // fp16 [NV][LD64]: V', transposed
+constexpr int N_S = 0;                            // fp16 [2][NV][LD128]: the state, transposed; even and odd chunks
+constexpr int N_V = N_S + 2 * NV * LD128 * 2;     // fp16 [NV][LD64]: V', transposed
 constexpr int INTER_LDS = N_V + NV * LD64 * 2;
 
 template <typename S>
@@ -624,7 +626,7 @@ __device__ __forceinline__ void store_state_elem4(bf16_t* p, const f32x4 v) {
 struct StateOperands {
     u32x4 w[4];                                   // rows 16 w + l % 16, keys 32 ks + 8 (l / 16) ..
     u32x4 k[2][2];                                // keys 32 w + 16 mt + l % 16, chunk rows 32 ks + 8 (l / 16) ..
-    uint2 u[NT];                                  // value 16 nt + l % 16, rows 16 w + 4 (l / 16) ..
+    uint2 u[NT];                                  // value column of (nt, l % 16), rows 16 w + 4 (l / 16) ..
     f32x4 e[2];                                   // keys 32 w + 16 mt + 4 (l / 16) ..
 };
 struct ReadoutOperands {
@@ -632,6 +634,11 @@ struct ReadoutOperands {
     u32x4 m[2];                                   // rows 16 w + l % 16, chunk rows 32 ks + 8 (l / 16) ..
 };
 constexpr int INTER_THREADS = 512;
+static_assert(NT == 2, "the value-column order below pairs two tiles");
+// Row m of value tile nt (of a workgroup's transposed state and V') is value column 8 (m / 4) + 4 nt + m % 4 of the
+// block: a read-out accumulator holds rows 4 g .. 4 g + 3 of both tiles, which is then eight consecutive values of
+// one output row, one 128-bit store.
+__device__ __forceinline__ int value_col(int nt, int m) { return 8 * (m >> 2) + 4 * nt + (m & 3); }
 
 // Pass 2: one head's NV value columns of one request through the chunks of the pass, in order. The state
 // S[128 keys][NV] lives in the MFMA accumulators of the state waves: wave w owns keys 32 w .. 32 w + 31. Only
@@ -659,7 +666,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
     const long long sbase = (state_off != nullptr ? state_off[b] : 0) + (long long)h * DV * DK;
     const int rl = 4 * (lane >> 4), cl = lane & 15;
 
-    uint16_t* Sl = reinterpret_cast<uint16_t*>(smem + N_S);
+    uint16_t* Sl2 = reinterpret_cast<uint16_t*>(smem + N_S);
     uint16_t* Vl = reinterpret_cast<uint16_t*>(smem + N_V);
     const unsigned char* wsh = ws + ((long long)b * H + h) * chunks * (long long)WS_BYTES;
     // Per-lane byte offsets of the fragments inside a chunk's workspace.
@@ -670,18 +677,18 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
     // (and every wave is done with the V' of the chunk before), after the second its V' is.
 
     if (state_wave) {
-        // the state: accS[mt][nt][r] = S[key 32 w + 16 mt + rl + r][value NV vb + 16 nt + cl]
+        // the state: accS[mt][nt][r] = S[key 32 w + 16 mt + rl + r][value NV vb + value_col(nt, cl)]
         f32x4 accS[2][NT];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 float v4[4];
-                load_state_elem4<S>(state_in + sbase + (long long)(NV * vb + SUB * nt + cl) * DK + 32 * wave + SUB * mt + rl, v4);
+                load_state_elem4<S>(state_in + sbase + (long long)(NV * vb + value_col(nt, cl)) * DK + 32 * wave + SUB * mt + rl, v4);
                 accS[mt][nt] = f32x4{v4[0], v4[1], v4[2], v4[3]};
             }
         const unsigned off_k = (unsigned)(WS_KGT + ((32 * wave + cl) * 32 + 8 * (lane >> 4)) * 2);  // + 1024 mt + 8192 ks
-        const unsigned off_u = (unsigned)(WS_UT + ((NV * vb + cl) * CH + SUB * wave + rl) * 2);     // + 2048 nt
+        const unsigned off_u = (unsigned)(WS_UT + ((NV * vb + value_col(0, cl)) * CH + SUB * wave + rl) * 2);   // + 512 nt
         const unsigned off_e = (unsigned)(WS_E + (32 * wave + rl) * 4);                             // + 64 mt
         // The loads of chunk C_ into operand set X_, one group at a time (each group is requested as soon as the
         // chunk two before it has used those registers). Unconditional: past the end they repeat the last chunk.
@@ -691,7 +698,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                        \
                 X_.w[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_W + off_a + 4096 * ks);                          \
             _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                        \
-                X_.u[nt] = *reinterpret_cast<const uint2*>(src_ + off_u + 2048 * nt);                                \
+                X_.u[nt] = *reinterpret_cast<const uint2*>(src_ + off_u + 512 * nt);                                 \
         }
 #define KDA_LOAD_KE(X_, C_)                                                                                         \
         {                                                                                                           \
@@ -705,6 +712,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
         // Chunk c with the operands in x; each group of x is then requested again for chunk c + 2.
         auto chunk_step = [&](const int c, StateOperands& x) __attribute__((always_inline)) {
             const int c2 = min(c + 2, nch - 1);
+            uint16_t* Sl = Sl2 + (c & 1) * (NV * LD128);
             // S^T (fp16) for the products of the chunk
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
@@ -783,11 +791,11 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
-                store_state_elem4(state_out + sbase + (long long)(NV * vb + SUB * nt + cl) * DK + 32 * wave + SUB * mt + rl,
+                store_state_elem4(state_out + sbase + (long long)(NV * vb + value_col(nt, cl)) * DK + 32 * wave + SUB * mt + rl,
                                   accS[mt][nt]);
     } else {
-        // rows of `out` that start on 8-byte boundaries take four values per store
-        const bool wide_out = ((reinterpret_cast<size_t>(out) | (size_t)(out_stride * 2)) & 7) == 0;
+        // rows of `out` that start on 16-byte boundaries take eight values per store
+        const bool wide_out = ((reinterpret_cast<size_t>(out) | (size_t)(out_stride * 2)) & 15) == 0;
 #define KDA_LOAD_QM(X_, C_)                                                                                         \
         {                                                                                                           \
             const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
@@ -796,40 +804,50 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                        \
                 X_.m[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_M + off_a + 4096 * ks);                          \
         }
+        // The read-out of a chunk starts after the chunk's second barrier, when both the state and V' are in LDS and
+        // the state waves are done with their long reads of the state; the rows are stored while the state waves
+        // work between the next chunk's barriers.
+        f32x4 accY[NT];
+        int st_c = -1;                            // the chunk whose read-out is in accY, not yet stored
+        auto store_rows = [&]() __attribute__((always_inline)) {
+            const int nrows = min(CH, left - st_c * CH);
+            if (SUB * wave + cl < nrows) {
+                // accY[nt][r] = y[row 16 w + cl][value NV vb + 2 rl + 4 nt + r]
+                bf16_t* orow = out + (rr.row0 + sub0 + st_c * CH + SUB * wave + cl) * out_stride + h * DV + NV * vb + 2 * rl;
+                const u32x4 y8 = {f2bf2(accY[0][0], accY[0][1]), f2bf2(accY[0][2], accY[0][3]),
+                                  f2bf2(accY[1][0], accY[1][1]), f2bf2(accY[1][2], accY[1][3])};
+                if (wide_out) *reinterpret_cast<u32x4*>(orow) = y8;
+                else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        orow[2 * e] = (bf16_t)(y8[e] & 0xffffu);
+                        orow[2 * e + 1] = (bf16_t)(y8[e] >> 16);
+                    }
+                }
+            }
+        };
         auto chunk_step = [&](const int c, ReadoutOperands& x) __attribute__((always_inline)) {
-            const int nrows = min(CH, left - c * CH);
             const int c2 = min(c + 2, nch - 1);
+            const uint16_t* Sl = Sl2 + (c & 1) * (NV * LD128);
+            __syncthreads();
+            if (st_c >= 0) store_rows();
             __syncthreads();
             // Y^T = S^T Qg^T + V'^T M^T: the state and V' on the row side of the tiles, so that a lane ends up with
             // four consecutive values of one row and stores them as one 8-byte piece
-            f32x4 accY[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) accY[nt] = zero;
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    accY[nt] = mfma_f16(frag(Sl, LD128, SUB * nt, 32 * ks, lane), as_u4(x.q[ks]), accY[nt]);
-            __syncthreads();
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
                     accY[nt] = mfma_f16(frag(Vl, LD64, SUB * nt, 32 * ks, lane), as_u4(x.m[ks]), accY[nt]);
-            KDA_LOAD_QM(x, c2)
-            if (SUB * wave + cl < nrows) {
-                // accY[nt][r] = y[row 16 w + cl][value NV vb + 16 nt + rl + r]
-                bf16_t* orow = out + (rr.row0 + sub0 + c * CH + SUB * wave + cl) * out_stride + h * DV + NV * vb + rl;
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const uint2 y4 = make_uint2(f2bf2(accY[nt][0], accY[nt][1]), f2bf2(accY[nt][2], accY[nt][3]));
-                    if (wide_out) *reinterpret_cast<uint2*>(orow + SUB * nt) = y4;
-                    else {
-                        orow[SUB * nt] = (bf16_t)(y4.x & 0xffffu); orow[SUB * nt + 1] = (bf16_t)(y4.x >> 16);
-                        orow[SUB * nt + 2] = (bf16_t)(y4.y & 0xffffu); orow[SUB * nt + 3] = (bf16_t)(y4.y >> 16);
-                    }
-                }
-            }
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    accY[nt] = mfma_f16(frag(Sl, LD128, SUB * nt, 32 * ks, lane), as_u4(x.q[ks]), accY[nt]);
+            KDA_LOAD_QM(x, c2)
+            st_c = c;
         };
         if (nch > 0) {
             ReadoutOperands xa, xb;
@@ -843,6 +861,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
                 chunk_step(c + 1, xb);
             }
             if (c < nch) chunk_step(c, xa);
+            store_rows();
         }
 #undef KDA_LOAD_QM
     }
@@ -989,8 +1008,7 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
     unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
     // 128-bit input staging needs every q | k | v and gate row segment on a 16-byte boundary (the model's strides
     // are); other layouts take the 16-bit path. Conv-window offsets are device data: whole windows keep alignment.
-    const int vec = aligned16(p) && aligned16(a) && aligned16(conv) && (p_stride % 8 == 0) && (a_stride % 8 == 0) &&
-                    (heads % 1 == 0);
+    const int vec = aligned16(p) && aligned16(a) && aligned16(conv) && (p_stride % 8 == 0) && (a_stride % 8 == 0);
     const int step = (int)chunks * CH;
     for (int sub0 = 0; sub0 == 0 || sub0 < max_rows; sub0 += step) {
         if (max_rows > 0) {
