@@ -158,6 +158,23 @@ __device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
 }
 
+// A 16 x 16 transpose on the matrix core. Every lane gives four fp16 values of its row (lane l: row l % 16, the
+// values at positions 4 (l / 16) .. + 3 of the row's sixteen); the product with the identity comes back in the
+// accumulator layout, in which lane l holds position l % 16 of rows 4 (l / 16) .. + 3: four consecutive rows of one
+// column, which is what a store into a [column][row] matrix wants. Exact: every sum has one nonzero term.
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4 transpose16(uint32_t v01, uint32_t v23, uint2 identity) {
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, make_uint2(v01, v23)),
+                                                 __builtin_bit_cast(f16x4, identity), zero, 0, 0, 0);
+}
+__device__ __forceinline__ uint2 transpose_identity(int lane) {   // rows 4 (l / 16) .. + 3 of column l % 16 of I
+    const int n = lane & 15, k0 = 4 * (lane >> 4);
+    const uint32_t one = 0x3c00u;
+    return make_uint2((k0 == n ? one : 0u) | (k0 + 1 == n ? one << 16 : 0u),
+                      (k0 + 2 == n ? one : 0u) | (k0 + 3 == n ? one << 16 : 0u));
+}
+
 // Pass 1: the chunks of one head of one request, everything that does not need the state, into their workspace
 // slots. Wave w owns sub-chunk w of a chunk (rows 16 w .. 16 w + 15); in the elementwise phases lane l holds row
 // l % 16 and 32 channels of it: with g = l / 16, the four pieces of eight channels 32 p + 8 g .. + 7, p = 0..3 (the
@@ -227,6 +244,10 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     asm volatile("" : "+v"(t));
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63;
     const int i = lane & 15, g = lane >> 4;       // this lane's row of the sub-chunk and its set of 32 channels
+    // what the lane holds after a transpose16: position cl_t (of the sixteen values the four lanes of a row put in:
+    // lane group cl_t / 4, its value cl_t % 4) of rows rl_t .. rl_t + 3 of the sub-chunk
+    const int cl_t = lane & 15, rl_t = 4 * (lane >> 4);
+    const uint2 ident = transpose_identity(lane);
     const int r0 = sub0 + c * CH;                 // the chunk's first row inside the request
     const int n = min(CH, rr.rows - r0);          // its real rows
     if (n <= 0) break;
@@ -265,6 +286,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 for (int it = 0; it < 12; ++it) halo[it] = load8<VEC>(hsrc + (long long)(it >> 2) * H * DK + 32 * (it & 3));
             }
         }
+        uint32_t vh[2];
 #pragma unroll
         for (int it = 0; it < 12; ++it) {
             const int seg = it >> 2, p = it & 3;
@@ -290,9 +312,13 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 if (seg == 0) { qr[4 * p + d] = pair; ssq = dot2_bf16(pair, pair, ssq); }
                 if (seg == 1) { kr[4 * p + d] = pair; ssk = dot2_bf16(pair, pair, ssk); }
                 if (seg == 2) {
-                    const float r0f = __uint_as_float(pair << 16), r1f = __uint_as_float(pair & 0xffff0000u);
-                    VT[(32 * p + 8 * g + 2 * d) * LD64 + R] = f2h(r0f);
-                    VT[(32 * p + 8 * g + 2 * d + 1) * LD64 + R] = f2h(r1f);
+                    // v as fp16, transposed into VT four rows at a time: two words are four values of the row
+                    vh[d & 1] = pack_h2(__uint_as_float(pair << 16), __uint_as_float(pair & 0xffff0000u));
+                    if (d & 1) {
+                        const f32x4 x = transpose16(vh[0], vh[1], ident);
+                        *reinterpret_cast<uint2*>(VT + (32 * p + 8 * (cl_t >> 2) + 4 * (d >> 1) + (cl_t & 3)) * LD64 +
+                                                  SUB * wave + rl_t) = make_uint2(pack_h2(x[0], x[1]), pack_h2(x[2], x[3]));
+                    }
                 }
             }
         }
@@ -365,30 +391,33 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // (G_0: the sub-chunk's first row, so that fifteen rows of decay bound the exponent), col2 = e^{G_15 - G_i}.
     // The diagonal tiles of L and M take k ep, q ep (rows) and k / ep (columns) straight from registers, four
     // channels per f32 MFMA (one per lane group).
-    const int rl = 4 * (lane >> 4), cl = lane & 15;   // an accumulator holds rows rl..rl+3 of column cl of a tile
+    // The tiles are computed transposed (column side first in the MFMA), so an accumulator holds columns rl..rl+3 of
+    // row cl of a tile: four consecutive elements of a row of L or M, one store.
+    const int rl = 4 * (lane >> 4), cl = lane & 15;
     uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
     // Store a finished tile at block (rb, cb). L = beta_i * acc: a diagonal block (strictly lower) in f32 for the
     // inversion, a block below the diagonal negated in fp16 as an MFMA operand of the block solve. M (lower with
     // the diagonal) goes to the workspace.
     auto put_L = [&](f32x4 acc, int rb, int cb) {
+        const int gi = SUB * rb + cl, gj = SUB * cb + rl;
+        const float bi = beta_s[gi];
+        if (rb == cb) {
+            f32x4 v;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int li = rl + r, gi = SUB * rb + li, gj = SUB * cb + cl;
-            const float v = beta_s[gi] * acc[r];
-            if (rb == cb) {
-                Ld[(SUB * rb + li) * LDD + cl] = cl < li ? v : 0.0f;
-                Ln[gi * LD64 + gj] = 0;
-            } else {
-                Ln[gi * LD64 + gj] = f2h(-v);
-            }
+            for (int r = 0; r < 4; ++r) v[r] = rl + r < cl ? bi * acc[r] : 0.0f;
+            *reinterpret_cast<f32x4*>(Ld + gi * LDD + rl) = v;
+            *reinterpret_cast<uint2*>(Ln + gi * LD64 + gj) = make_uint2(0u, 0u);
+        } else {
+            *reinterpret_cast<uint2*>(Ln + gi * LD64 + gj) =
+                make_uint2(pack_h2(-(bi * acc[0]), -(bi * acc[1])), pack_h2(-(bi * acc[2]), -(bi * acc[3])));
         }
     };
     auto put_M = [&](f32x4 acc, int rb, int cb) {
+        const int gi = SUB * rb + cl, gj = SUB * cb + rl;
+        float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int gi = SUB * rb + rl + r, gj = SUB * cb + cl;
-            Mg[panel_index(CH, gi, gj)] = f2h((rb != cb || gj <= gi) ? acc[r] : 0.0f);
-        }
+        for (int r = 0; r < 4; ++r) v[r] = (rb != cb || gj + r <= gi) ? acc[r] : 0.0f;
+        *reinterpret_cast<uint2*>(Mg + panel_index(CH, gi, gj)) = make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
     };
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
     float ke1[32], qe1[32];                       // k e^{G_i}, q e^{G_i}: the row side of the tiles left of the diagonal
@@ -401,7 +430,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         for (int p = 0; p < 4; ++p) {
             const f32x4 b0 = *reinterpret_cast<const f32x4*>(eB + 32 * p), b1 = *reinterpret_cast<const f32x4*>(eB + 32 * p + 4);
             const f32x4 s0 = *reinterpret_cast<const f32x4*>(eSuf + 32 * p), s1 = *reinterpret_cast<const f32x4*>(eSuf + 32 * p + 4);
-            float qg[8], kc[8];
+            float qg[8], kc[8], ket[8], kgt[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const int ch = 8 * p + e;
@@ -415,15 +444,24 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 const float qraw = (ch & 1) ? __uint_as_float(qr[ch >> 1] & 0xffff0000u) : __uint_as_float(qr[ch >> 1] << 16);
                 const float kh = kraw * kinv, qh = qraw * qinv;
                 const float kcd = kh * rp;
-                accL = __builtin_amdgcn_mfma_f32_16x16x4f32(kh * ep, kcd, accL, 0, 0, 0);
-                accM = __builtin_amdgcn_mfma_f32_16x16x4f32(qh * ep, kcd, accM, 0, 0, 0);
+                accL = __builtin_amdgcn_mfma_f32_16x16x4f32(kcd, kh * ep, accL, 0, 0, 0);
+                accM = __builtin_amdgcn_mfma_f32_16x16x4f32(kcd, qh * ep, accM, 0, 0, 0);
                 ke1[ch] = kh * e1;
                 qe1[ch] = qh * e1;
                 const float fb = e < 4 ? b0[e] : b1[e - 4], fs = e < 4 ? s0[e] : s1[e - 4];
-                keT[(32 * p + 8 * g + e) * LD64 + R] = f2h(ke1[ch] * fb);
-                kgT[panel_index(DK, 32 * p + 8 * g + e, R)] = f2h(kh * col2 * fs);
+                ket[e] = ke1[ch] * fb;
+                kgt[e] = kh * col2 * fs;
                 qg[e] = qe1[ch] * fb;
                 kc[e] = kh * col2;
+            }
+            // k e^G into LDS and Kg into the workspace, both [key][row]: transposed four rows at a time
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                const int key = 32 * p + 8 * (cl_t >> 2) + 4 * hf + (cl_t & 3);
+                const f32x4 x = transpose16(pack_h2(ket[4 * hf], ket[4 * hf + 1]), pack_h2(ket[4 * hf + 2], ket[4 * hf + 3]), ident);
+                *reinterpret_cast<uint2*>(keT + key * LD64 + SUB * wave + rl_t) = make_uint2(pack_h2(x[0], x[1]), pack_h2(x[2], x[3]));
+                const f32x4 y = transpose16(pack_h2(kgt[4 * hf], kgt[4 * hf + 1]), pack_h2(kgt[4 * hf + 2], kgt[4 * hf + 3]), ident);
+                *reinterpret_cast<uint2*>(kgT + panel_index(DK, key, SUB * wave + rl_t)) = make_uint2(pack_h2(y[0], y[1]), pack_h2(y[2], y[3]));
             }
             *reinterpret_cast<u32x4*>(wsc + WS_QG + panel_index(CH, R, 32 * p + 8 * g) * 2) =
                 u32x4{pack_h2(qg[0], qg[1]), pack_h2(qg[2], qg[3]), pack_h2(qg[4], qg[5]), pack_h2(qg[6], qg[7])};
@@ -456,8 +494,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             }
             const uint4 ka = make_uint4(pack_h2(ak[0], ak[1]), pack_h2(ak[2], ak[3]), pack_h2(ak[4], ak[5]), pack_h2(ak[6], ak[7]));
             const uint4 qa = make_uint4(pack_h2(aq[0], aq[1]), pack_h2(aq[2], aq[3]), pack_h2(aq[4], aq[5]), pack_h2(aq[6], aq[7]));
-            accL = mfma_f16(ka, bcol, accL);
-            accM = mfma_f16(qa, bcol, accM);
+            accL = mfma_f16(bcol, ka, accL);
+            accM = mfma_f16(bcol, qa, accM);
         }
         put_L(accL, wave, cb);
         put_M(accM, wave, cb);
