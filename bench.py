@@ -179,6 +179,19 @@ def bench_decode(steps, warmup, stream, cpu=True):
     ms_two = timed(step_two_launches, steps, max(1, warmup // 2), stream)
     ms_chain = timed(chains_only, steps, max(1, warmup // 2), stream) / layers
     state_bytes = 2 * batch * n * 2                      # read + write of 16 bf16 states: 67,108,864 B
+    # What this box moves for the same traffic with no arithmetic behind it: the same entry point with requests of
+    # zero rows copies every slot's state to `state_out` (here the next layer's pool), same workgroups, same
+    # nontemporal accesses, 32 MiB read and 32 MiB written per launch.
+    cu0 = torch.zeros(batch + 1, dtype=torch.int32, device=DEV)
+    copy_args = [(heads, batch, ptr(cu0), *rows.row_args(), ptr(convs[l]), ptr(coff), ptr(layer.conv_w), ptr(pools[l]),
+                  ptr(pools[(l + 1) % layers]), ptr(soff), *layer.args(), *rows.out_args(), None, None, None, None, st)
+                 for l in range(layers)]
+
+    def copies_only():
+        for l in range(layers):
+            check(chain_fn(*copy_args[l]), "chain (zero rows)")
+
+    ms_copy = timed(copies_only, steps, max(1, warmup // 2), stream) / layers
     res = {
         "ms_per_step": ms_step,
         "state_GBps": layers * state_bytes / (ms_step * 1e-3) / 1e9,
@@ -188,7 +201,9 @@ def bench_decode(steps, warmup, stream, cpu=True):
                      "unit": "GB/s", "frac": state_bytes / (ms_chain * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": TRAFFIC_BYTES["decode_chain"],
                      "kernel": "chain_kernel<bf16>", "bytes_per_launch": state_bytes,
-                     "us_per_launch": ms_chain * 1e3},
+                     "us_per_launch": ms_chain * 1e3,
+                     "same_traffic_copy": {"us_per_launch": ms_copy * 1e3, "GBps": state_bytes / (ms_copy * 1e-3) / 1e9,
+                                           "what": "zero-row requests: each slot's state copied to another pool"}},
     }
     if cpu:
         from oracle import kda_oracle as o
