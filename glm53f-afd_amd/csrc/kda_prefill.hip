@@ -1,5 +1,6 @@
 // KDA chunked prefill on gfx950: the delta rule over a prompt segment in the chunked (WY/UT) form, with every
-// GEMM-shaped step on the matrix cores (v_mfma_f32_16x16x32_f16 and, for a few tiles, v_mfma_f32_16x16x4_f32).
+// GEMM-shaped step on the matrix cores (v_mfma_f32_16x16x32_f16; for a few tiles v_mfma_f32_16x16x4_f32; and
+// v_mfma_f32_16x16x16_f16 against the identity as a register transpose).
 //
 // The algebra is the reference's chunk form (crates/glm53f-kda/src/chunked.rs:67-198; kernel counterpart
 // kda_prefill.cu:95-538 with 16-row chunks on CUDA cores). Here a chunk is 64 rows in four sub-chunks of 16.
@@ -15,9 +16,9 @@
 // Everything that feeds the state is fp16 or f32. Only the diagonal 16x16 blocks of T are formed (in f32);
 // W and U come from a block forward substitution on [k e^G | v] with MFMA tiles (see intra_kernel).
 //
-// Kernels per pass: intra_kernel (one workgroup per chunk, head, request: prologue + L, M, T, W, U, Qg, Kg into
-// the workspace), inter_kernel (one workgroup per head, value-column block, request: the state in MFMA
-// accumulators across the chunks of the pass), then norm_kernel (gated RMSNorm in place, and the conv windows'
+// Kernels per pass: intra_kernel (one workgroup per two chunks of a head and request: prologue + L, M, T, W, U, Qg,
+// Kg into the workspace), inter_kernel (one workgroup per head, value-column block, request: the state in MFMA
+// accumulators across the chunks of the pass); then, once per call, norm_kernel (gated RMSNorm in place, and the conv windows'
 // advance).
 
 #include "kda_common.h"
