@@ -86,11 +86,11 @@ constexpr int I_LD = I_LN + CH * LD64 * 2;        // f32 [4][16][LDD]: the diago
 constexpr int I_KCE = I_LD + 4 * SUB * LDD * 4;   // fp16 [3][16][LD128]: k e^{G_end - G} of sub-chunks 0..2, row major
 constexpr int I_Z = I_KCE;                        //   later fp16 [16 column tiles][16][LDZ]: a tile of Z on its way back
 constexpr int I_FAC = I_KCE + 3 * SUB * LD128 * 2;  // f32 [NFAC][128]
-constexpr int I_TT = I_FAC;                       //   later fp16 [64][LDT]: row 16 a + i holds [T_aa diag(beta) | T_aa][i][0..32)
+constexpr int I_TT = I_LD;                        //   later fp16 [64][LDT]: row 16 a + i holds [T_aa diag(beta) | T_aa][i][0..32)
 constexpr int INTRA_LDS = I_FAC + NFAC * DK * 4;
 constexpr int INTRA_CPW = 2;                      // consecutive chunks of a head per intra workgroup
 static_assert(16 * SUB * LDZ * 2 <= 3 * SUB * LD128 * 2, "Z fits the region of the column operands");
-static_assert(CH * LDT * 2 <= NFAC * DK * 4, "TT fits the region of the factors");
+static_assert(LDT * 2 == LDD * 4, "a row of TT takes the place of the row of the diagonal block it comes from");
 static_assert(2 * INTRA_LDS <= 160 * 1024, "two intra workgroups per CU");
 
 // Factors e^{sum of whole sub-chunks' log decay}, per key channel: 0..3 = e^{G before sub-chunk a};
@@ -266,6 +266,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             av[p] = load8<VEC>(arow + 32 * p);
         }
     }
+    // the beta logit of row t (lanes of wave 0), requested now as well: its use sits right before a barrier
+    const bf16_t b_raw = P[(rr.row0 + r0 + min((int)(t & (CH - 1)), n - 1)) * p_stride + b_off + h];
 
     // ---- conv + SiLU with one bf16 rounding (q, k stay in registers; v goes to VT as fp16, exact but for values
     // below 2^-14), and the sums of squares for the L2 norms. Rows past the request's end are not masked: their
@@ -359,7 +361,6 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         }
     }
     if (t < CH) {
-        const bf16_t b_raw = t < n ? P[(rr.row0 + r0 + t) * p_stride + b_off + h] : (bf16_t)0;
         beta_s[t] = t < n ? bfround(fast_sigmoid(bf2f(b_raw))) : 0.0f;
     }
     __syncthreads();
@@ -475,53 +476,26 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         put_M(accM, wave, wave);
     }
     __syncthreads();                              // the column operands of every sub-chunk are in place
-    // tiles left of the diagonal: rows of sub-chunk `wave` against the columns of sub-chunk cb. In MFMA step s lane
-    // group g supplies channels 32 s + 8 g .. + 7 on both sides (which k a lane supplies is free as long as both
-    // operands agree).
-#pragma unroll 1
-    for (int cb = 0; cb < wave; ++cb) {
-        const float* df = fac + factor_index(wave, cb) * DK + 8 * g;
-        const uint16_t* kcol = KcE + (cb * SUB + i) * LD128 + 8 * g;
-        f32x4 accL = zero, accM = zero;
+    uint16_t* TT = reinterpret_cast<uint16_t*>(smem + I_TT);
+    if (wave == 0) {
+        // Sub-chunk 0 has no tiles left of its diagonal, so while the other waves compute theirs wave 0 does what
+        // needs the diagonal blocks only.
+        // M and -L above the block diagonal are zero: blocks (0,1), (0,2), (0,3), (1,2), (1,3), (2,3), in 128-bit
+        // pieces (two per row of a block)
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const f32x4 d0 = *reinterpret_cast<const f32x4*>(df + 32 * s), d1 = *reinterpret_cast<const f32x4*>(df + 32 * s + 4);
-            const uint4 bcol = *reinterpret_cast<const uint4*>(kcol + 32 * s);
-            float ak[8], aq[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float f = e < 4 ? d0[e] : d1[e - 4];
-                ak[e] = ke1[8 * s + e] * f;
-                aq[e] = qe1[8 * s + e] * f;
-            }
-            const uint4 ka = make_uint4(pack_h2(ak[0], ak[1]), pack_h2(ak[2], ak[3]), pack_h2(ak[4], ak[5]), pack_h2(ak[6], ak[7]));
-            const uint4 qa = make_uint4(pack_h2(aq[0], aq[1]), pack_h2(aq[2], aq[3]), pack_h2(aq[4], aq[5]), pack_h2(aq[6], aq[7]));
-            accL = mfma_f16(bcol, ka, accL);
-            accM = mfma_f16(bcol, qa, accM);
-        }
-        put_L(accL, wave, cb);
-        put_M(accM, wave, cb);
-    }
-    __syncthreads();                              // L is complete; the factors and column operands are dead
-    // M and -L above the block diagonal are zero: blocks (0,1), (0,2), (0,3), (1,2), (1,3), (2,3)
-    {
-        uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
-        // by waves 1 to 3: wave 0 goes straight to the inversion below
-        for (int e = t - 64; e >= 0 && e < 6 * 256; e += THREADS - 64) {
-            const int blk = e >> 8, r = (e >> 4) & 15, cc = e & 15;
+        for (int it = 0; it < 3; ++it) {
+            const int e = lane + 64 * it, blk = e >> 5, r = (e >> 1) & 15, half = e & 1;
             const int rb = blk < 3 ? 0 : (blk < 5 ? 1 : 2);
             const int cb = blk < 3 ? blk + 1 : (blk < 5 ? blk - 1 : 3);
-            Mg[panel_index(CH, SUB * rb + r, SUB * cb + cc)] = 0;
-            Ln[(SUB * rb + r) * LD64 + SUB * cb + cc] = 0;
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4*>(Mg + panel_index(CH, SUB * rb + r, SUB * cb + 8 * half)) = z;
+            *reinterpret_cast<u32x4*>(Ln + (SUB * rb + r) * LD64 + SUB * cb + 8 * half) = z;
         }
-    }
-
-    // ---- the diagonal blocks of T = (I + L)^-1 in f32 by forward substitution: lane (a, j) solves column j of
-    // block a and leaves it as fp16 operands, scaled by beta_j (T' = T diag(beta)) and plain.
-    uint16_t* TT = reinterpret_cast<uint16_t*>(smem + I_TT);
-    if (t < CH) {
-        const int a = t >> 4, j = t & 15;
-        const float bj = beta_s[t];
+        // ---- the diagonal blocks of T = (I + L)^-1 in f32 by forward substitution: lane (a, j) solves column j of
+        // block a and leaves it as fp16 operands, scaled by beta_j (T' = T diag(beta)) and plain. TT takes the place
+        // of the blocks it is computed from: every lane has its block in registers before any lane writes.
+        const int a = lane >> 4, j = lane & 15;
+        const float bj = beta_s[lane];
         // the block's strictly lower triangle into registers (rows as 128-bit pieces), then the substitution
         // column by column: once x[m] is known every later row takes its term, sixteen independent chains
         float l[SUB][SUB];
@@ -542,13 +516,44 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
             for (int i = m + 1; i < SUB; ++i) acc[i] = __builtin_fmaf(l[i][m], x[m], acc[i]);
         }
+        // the reads of Ld above are complete (their values are used) and stay ahead of the writes below
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int i = 0; i < SUB; ++i) {
             TT[(SUB * a + i) * LDT + j] = f2h(x[i] * bj);
             TT[(SUB * a + i) * LDT + SUB + j] = f2h(x[i]);
         }
+    } else {
+        // tiles left of the diagonal: rows of sub-chunk `wave` against the columns of sub-chunk cb. In MFMA step s
+        // lane group g supplies channels 32 s + 8 g .. + 7 on both sides (which k a lane supplies is free as long as
+        // both operands agree).
+#pragma unroll 1
+        for (int cb = 0; cb < wave; ++cb) {
+            const float* df = fac + factor_index(wave, cb) * DK + 8 * g;
+            const uint16_t* kcol = KcE + (cb * SUB + i) * LD128 + 8 * g;
+            f32x4 accL = zero, accM = zero;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const f32x4 d0 = *reinterpret_cast<const f32x4*>(df + 32 * s), d1 = *reinterpret_cast<const f32x4*>(df + 32 * s + 4);
+                const uint4 bcol = *reinterpret_cast<const uint4*>(kcol + 32 * s);
+                float ak[8], aq[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float f = e < 4 ? d0[e] : d1[e - 4];
+                    ak[e] = ke1[8 * s + e] * f;
+                    aq[e] = qe1[8 * s + e] * f;
+                }
+                const uint4 ka = make_uint4(pack_h2(ak[0], ak[1]), pack_h2(ak[2], ak[3]), pack_h2(ak[4], ak[5]), pack_h2(ak[6], ak[7]));
+                const uint4 qa = make_uint4(pack_h2(aq[0], aq[1]), pack_h2(aq[2], aq[3]), pack_h2(aq[4], aq[5]), pack_h2(aq[6], aq[7]));
+                accL = mfma_f16(bcol, ka, accL);
+                accM = mfma_f16(bcol, qa, accM);
+            }
+            put_L(accL, wave, cb);
+            put_M(accM, wave, cb);
+        }
     }
-    __syncthreads();
+    __syncthreads();                              // L and TT are complete; the factors and column operands are dead
     if (c + 1 < min(chunks, c_first + INTRA_CPW)) load_own(r0 + CH);   // the next chunk's rows
 
     // ---- W = T' (k e^G) and U = T' v without the blocks of T below the diagonal: block forward substitution on
@@ -598,16 +603,18 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 }
             }
             if (wave < 2) {
-                // key columns: X^T tile [16 keys][16 rows], so a lane ends with four consecutive keys of one row
-                // of W [row][key] for the workspace; back into R^T as four 16-bit pieces
-                f32x4 x[4];
+                // key columns, both ways round: the X^T tile [16 keys][16 rows] leaves a lane four consecutive keys of
+                // one row of W [row][key] for the workspace, the X tile four consecutive rows of one key for R^T
+                f32x4 x[4], xr[4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) x[q] = mfma_f16(rz[q], tt, zero);
+                for (int q = 0; q < 4; ++q) {
+                    x[q] = mfma_f16(rz[q], tt, zero);
+                    xr[q] = mfma_f16(tt, rz[q], zero);
+                }
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int ct = 4 * wave + q;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) RT[(SUB * ct + rl + r) * LD64 + SUB * a + cl] = f2h(x[q][r]);
+                    *reinterpret_cast<uint2*>(RT + (SUB * ct + cl) * LD64 + SUB * a + rl) = pack4(xr[q]);
                     *reinterpret_cast<uint2*>(wsc + WS_W + panel_index(CH, SUB * a + cl, SUB * ct + rl) * 2) = pack4(x[q]);
                 }
             } else {
