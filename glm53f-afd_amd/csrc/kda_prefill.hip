@@ -210,6 +210,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     float* Ld = reinterpret_cast<float*>(smem + I_LD);
     uint16_t* KcE = reinterpret_cast<uint16_t*>(smem + I_KCE);
     float* fac = reinterpret_cast<float*>(smem + I_FAC);
+    float* first = reinterpret_cast<float*>(smem + I_KCE);          // [4][128]: until the column operands go there
 
     // the head's conv weights and dt_bias, once (the first barrier of the chunk loop publishes them... they are
     // read before it, so one barrier here)
@@ -359,41 +360,50 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             for (int p = 0; p < 8; ++p)
                 *reinterpret_cast<f32x4*>(tot + wave * DK + 32 * (p >> 1) + 8 * g + 4 * (p & 1)) = f32x4{G[4 * p], G[4 * p + 1], G[4 * p + 2], G[4 * p + 3]};
         }
+        if (i == 0) {                             // G_0: the first row's own gate
+#pragma unroll
+            for (int p = 0; p < 8; ++p)
+                *reinterpret_cast<f32x4*>(first + wave * DK + 32 * (p >> 1) + 8 * g + 4 * (p & 1)) = f32x4{G[4 * p], G[4 * p + 1], G[4 * p + 2], G[4 * p + 3]};
+        }
     }
     if (t < CH) {
         beta_s[t] = t < n ? bfround(fast_sigmoid(bf2f(b_raw))) : 0.0f;
     }
     __syncthreads();
-    // the factors between sub-chunks, one channel per lane; e^{G_last} goes to the workspace
+    // the factors between sub-chunks, one channel per lane; e^{G_last} goes to the workspace. The row side of the
+    // tiles is kept relative to its sub-chunk's first row (k e^{G_i - G_0}), so the factors that meet it carry
+    // e^{G_0} of their sub-chunk (u) on top of the decay between the sub-chunks.
     {
         const int d = t & (DK - 1);
         const float t0 = tot[d], t1 = tot[DK + d], t2 = tot[2 * DK + d], t3 = tot[3 * DK + d];
+        const float u0 = first[d], u1 = first[DK + d], u2 = first[2 * DK + d], u3 = first[3 * DK + d];
         if (t < DK) {
-            fac[0 * DK + d] = 1.0f;
-            fac[1 * DK + d] = __builtin_amdgcn_exp2f(t0);
-            fac[2 * DK + d] = __builtin_amdgcn_exp2f(t0 + t1);
-            fac[3 * DK + d] = __builtin_amdgcn_exp2f(t0 + t1 + t2);
+            fac[0 * DK + d] = __builtin_amdgcn_exp2f(u0);
+            fac[1 * DK + d] = __builtin_amdgcn_exp2f(t0 + u1);
+            fac[2 * DK + d] = __builtin_amdgcn_exp2f(t0 + t1 + u2);
+            fac[3 * DK + d] = __builtin_amdgcn_exp2f(t0 + t1 + t2 + u3);
             reinterpret_cast<float*>(wsc + WS_E)[d] = __builtin_amdgcn_exp2f(t0 + t1 + t2 + t3);
             fac[4 * DK + d] = __builtin_amdgcn_exp2f(t1 + t2 + t3);
             fac[5 * DK + d] = __builtin_amdgcn_exp2f(t2 + t3);
         } else {
             fac[6 * DK + d] = __builtin_amdgcn_exp2f(t3);
             fac[7 * DK + d] = 1.0f;
-            fac[factor_index(1, 0) * DK + d] = 1.0f;
-            fac[factor_index(2, 0) * DK + d] = __builtin_amdgcn_exp2f(t1);
-            fac[factor_index(2, 1) * DK + d] = 1.0f;
-            fac[factor_index(3, 0) * DK + d] = __builtin_amdgcn_exp2f(t1 + t2);
-            fac[factor_index(3, 1) * DK + d] = __builtin_amdgcn_exp2f(t2);
-            fac[factor_index(3, 2) * DK + d] = 1.0f;
+            fac[factor_index(1, 0) * DK + d] = __builtin_amdgcn_exp2f(u1);
+            fac[factor_index(2, 0) * DK + d] = __builtin_amdgcn_exp2f(t1 + u2);
+            fac[factor_index(2, 1) * DK + d] = __builtin_amdgcn_exp2f(u2);
+            fac[factor_index(3, 0) * DK + d] = __builtin_amdgcn_exp2f(t1 + t2 + u3);
+            fac[factor_index(3, 1) * DK + d] = __builtin_amdgcn_exp2f(t2 + u3);
+            fac[factor_index(3, 2) * DK + d] = __builtin_amdgcn_exp2f(u3);
         }
     }
 
     __syncthreads();                              // the factors are in place
 
-    // ---- operands. Per element: e1 = e^{G_i} (from the sub-chunk's start), ep = e^{G_i - G_0} and its reciprocal
-    // (G_0: the sub-chunk's first row, so that fifteen rows of decay bound the exponent), col2 = e^{G_15 - G_i}.
+    // ---- operands. Per element: ep = e^{G_i - G_0} and its reciprocal (G_0: the sub-chunk's first row, so that
+    // fifteen rows of decay bound the exponent); e^{G_15 - G_i} is the last row's ep over the own one.
     // The diagonal tiles of L and M take k ep, q ep (rows) and k / ep (columns) straight from registers, four
-    // channels per f32 MFMA (one per lane group).
+    // channels per f32 MFMA (one per lane group); the same k ep, q ep are the row side of the other tiles and of
+    // k e^G and Qg, times factors that carry e^{G_0}.
     // The tiles are computed transposed (column side first in the MFMA), so an accumulator holds columns rl..rl+3 of
     // row cl of a tile: four consecutive elements of a row of L or M, one store.
     const int rl = 4 * (lane >> 4), cl = lane & 15;
@@ -423,7 +433,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         *reinterpret_cast<uint2*>(Mg + panel_index(CH, gi, gj)) = make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
     };
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-    float ke1[32], qe1[32];                       // k e^{G_i}, q e^{G_i}: the row side of the tiles left of the diagonal
+    float kep[32], qep[32];                       // k e^{G_i - G_0}, q e^{G_i - G_0}: the row side of every tile
     {
         f32x4 accL = zero, accM = zero;
         uint16_t* kgT = reinterpret_cast<uint16_t*>(wsc + WS_KGT);
@@ -439,23 +449,22 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 const int ch = 8 * p + e;
                 const float Gi = G[ch];
                 const float G0 = row_lane<0>(Gi);
-                const float e1 = __builtin_amdgcn_exp2f(Gi);
                 const float ep = __builtin_amdgcn_exp2f(Gi - G0);
                 const float rp = fast_rcp(ep);                  // e^{G_0 - G_i}, up to e^87
-                const float col2 = row_lane<SUB - 1>(ep) * rp;  // e^{G_15 - G_i}
+                const float last = row_lane<SUB - 1>(ep);       // e^{G_15 - G_0}
                 const float kraw = (ch & 1) ? __uint_as_float(kr[ch >> 1] & 0xffff0000u) : __uint_as_float(kr[ch >> 1] << 16);
                 const float qraw = (ch & 1) ? __uint_as_float(qr[ch >> 1] & 0xffff0000u) : __uint_as_float(qr[ch >> 1] << 16);
                 const float kh = kraw * kinv, qh = qraw * qinv;
                 const float kcd = kh * rp;
-                accL = __builtin_amdgcn_mfma_f32_16x16x4f32(kcd, kh * ep, accL, 0, 0, 0);
-                accM = __builtin_amdgcn_mfma_f32_16x16x4f32(kcd, qh * ep, accM, 0, 0, 0);
-                ke1[ch] = kh * e1;
-                qe1[ch] = qh * e1;
+                kep[ch] = kh * ep;
+                qep[ch] = qh * ep;
+                accL = __builtin_amdgcn_mfma_f32_16x16x4f32(kcd, kep[ch], accL, 0, 0, 0);
+                accM = __builtin_amdgcn_mfma_f32_16x16x4f32(kcd, qep[ch], accM, 0, 0, 0);
                 const float fb = e < 4 ? b0[e] : b1[e - 4], fs = e < 4 ? s0[e] : s1[e - 4];
-                ket[e] = ke1[ch] * fb;
-                kgt[e] = kh * col2 * fs;
-                qg[e] = qe1[ch] * fb;
-                kc[e] = kh * col2;
+                ket[e] = kep[ch] * fb;                          // k e^{G_i} from the chunk's start
+                qg[e] = qep[ch] * fb;
+                kc[e] = kcd * last;                             // k e^{G_15 - G_i}
+                kgt[e] = kc[e] * fs;
             }
             // k e^G into LDS and Kg into the workspace, both [key][row]: transposed four rows at a time
 #pragma unroll
@@ -541,8 +550,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float f = e < 4 ? d0[e] : d1[e - 4];
-                    ak[e] = ke1[8 * s + e] * f;
-                    aq[e] = qe1[8 * s + e] * f;
+                    ak[e] = kep[8 * s + e] * f;
+                    aq[e] = qep[8 * s + e] * f;
                 }
                 const uint4 ka = make_uint4(pack_h2(ak[0], ak[1]), pack_h2(ak[2], ak[3]), pack_h2(ak[4], ak[5]), pack_h2(ak[6], ak[7]));
                 const uint4 qa = make_uint4(pack_h2(aq[0], aq[1]), pack_h2(aq[2], aq[3]), pack_h2(aq[4], aq[5]), pack_h2(aq[6], aq[7]));
