@@ -338,7 +338,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // ---- gates: the cumulative log decay of the lane's row inside its sub-chunk, per channel
     float G[32];
     {
-        const uint32_t keep = R < n ? 0xffffffffu : 0u;    // a row past the end counts as g = 0
+        const float lower_r = R < n ? lower2 : 0.0f;       // a row past the end counts as g = 0
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const f32x4 d0 = *reinterpret_cast<const f32x4*>(dtb_s + 32 * p + 8 * g);
@@ -346,8 +346,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float dtb = e < 4 ? d0[e] : d1[e - 4];
-                const float gv = lower2 * fast_rcp(1.0f + __builtin_amdgcn_exp2f(__builtin_fmaf(gate_c, bf_at(av[p], e), dtb)));
-                float x = __uint_as_float(__float_as_uint(gv) & keep);
+                float x = lower_r * fast_rcp(1.0f + __builtin_amdgcn_exp2f(__builtin_fmaf(gate_c, bf_at(av[p], e), dtb)));
                 x += row_shr<1>(x);               // inclusive scan over the sixteen rows
                 x += row_shr<2>(x);
                 x += row_shr<4>(x);
@@ -567,7 +566,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
 
     // ---- W = T' (k e^G) and U = T' v without the blocks of T below the diagonal: block forward substitution on
     // R = [k e^G | v] (64 rows, 256 columns), held transposed in LDS ([column][row]: keT then VT) and solved in
-    // place, sixteen columns per tile, four tiles per wave, no barrier:
+    // place, sixteen columns per tile, four tiles per wave (two of keys, two of values: the key tiles cost a product
+    // and a store more), no barrier:
     //   Z_a = -sum_{b<a} L_ab X_b,   X_a = T'_aa R_a + T_aa Z_a.
     // R_a enters the last product unrounded (v is exact in fp16), so X is rounded once; Z, X_b and L are fp16.
     {
@@ -579,6 +579,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         auto pack4 = [](const f32x4 v) {
             return make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
         };
+        // the wave's column tiles: q = 0, 1 are key tiles 2 w + q, q = 2, 3 value tiles 8 + 2 w + q - 2
+        auto tile = [&](int q) { return q < 2 ? 2 * wave + q : 6 + 2 * wave + q; };
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const uint4 tt = frag(TT, LDT, SUB * a, 0, lane);
@@ -587,22 +589,22 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 f32x4 z[4];
                 const uint4 l0 = frag(Ln, LD64, SUB * a, 0, lane);
 #pragma unroll
-                for (int q = 0; q < 4; ++q) z[q] = mfma_f16(l0, frag(RT, LD64, SUB * (4 * wave + q), 0, lane), zero);
+                for (int q = 0; q < 4; ++q) z[q] = mfma_f16(l0, frag(RT, LD64, SUB * tile(q), 0, lane), zero);
                 if (a == 3) {
                     const uint4 l1 = frag(Ln, LD64, SUB * a, 32, lane);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) z[q] = mfma_f16(l1, frag(RT, LD64, SUB * (4 * wave + q), 32, lane), z[q]);
+                    for (int q = 0; q < 4; ++q) z[q] = mfma_f16(l1, frag(RT, LD64, SUB * tile(q), 32, lane), z[q]);
                 }
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
-                    *reinterpret_cast<uint2*>(Zs + ((4 * wave + q) * SUB + cl) * LDZ + rl) = pack4(z[q]);
+                    *reinterpret_cast<uint2*>(Zs + (tile(q) * SUB + cl) * LDZ + rl) = pack4(z[q]);
             }
             // [R_a | Z_a] of a column tile as an operand [16 columns][K = 32]: k < 16 is R_a (lanes 0..31), k >= 16
             // is Z_a (lanes 32..63): one read at a per-lane offset, no branch
             uint4 rz[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int ct = 4 * wave + q;
+                const int ct = tile(q);
                 const int off_r = I_KET + ((SUB * ct + cl) * LD64 + SUB * a + 8 * (lane >> 4)) * 2;
                 const int off_z = I_Z + ((ct * SUB + cl) * LDZ + 8 * ((lane >> 4) - 2)) * 2;
                 rz[q] = *reinterpret_cast<const uint4*>(smem + (lane < 32 ? off_r : off_z));
@@ -611,29 +613,21 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                     rz[q] = make_uint4(rz[q].x & keep, rz[q].y & keep, rz[q].z & keep, rz[q].w & keep);
                 }
             }
-            if (wave < 2) {
-                // key columns, both ways round: the X^T tile [16 keys][16 rows] leaves a lane four consecutive keys of
-                // one row of W [row][key] for the workspace, the X tile four consecutive rows of one key for R^T
-                f32x4 x[4], xr[4];
+            // key columns, both ways round: the X^T tile [16 keys][16 rows] leaves a lane four consecutive keys of one
+            // row of W [row][key] for the workspace, the X tile four consecutive rows of one key for R^T; value
+            // columns: the X tile [16 rows][16 values] only
+            f32x4 x[4], xt[2];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    x[q] = mfma_f16(rz[q], tt, zero);
-                    xr[q] = mfma_f16(tt, rz[q], zero);
-                }
+            for (int q = 0; q < 4; ++q) {
+                x[q] = mfma_f16(tt, rz[q], zero);
+                if (q < 2) xt[q] = mfma_f16(rz[q], tt, zero);
+            }
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int ct = 4 * wave + q;
-                    *reinterpret_cast<uint2*>(RT + (SUB * ct + cl) * LD64 + SUB * a + rl) = pack4(xr[q]);
-                    *reinterpret_cast<uint2*>(wsc + WS_W + panel_index(CH, SUB * a + cl, SUB * ct + rl) * 2) = pack4(x[q]);
-                }
-            } else {
-                // value columns: X tile [16 rows][16 values]: four consecutive rows of one value, one piece of R^T
-                f32x4 x[4];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) x[q] = mfma_f16(tt, rz[q], zero);
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    *reinterpret_cast<uint2*>(RT + (SUB * (4 * wave + q) + cl) * LD64 + SUB * a + rl) = pack4(x[q]);
+            for (int q = 0; q < 4; ++q) {
+                const int ct = tile(q);
+                *reinterpret_cast<uint2*>(RT + (SUB * ct + cl) * LD64 + SUB * a + rl) = pack4(x[q]);
+                if (q < 2)
+                    *reinterpret_cast<uint2*>(wsc + WS_W + panel_index(CH, SUB * a + cl, SUB * ct + rl) * 2) = pack4(xt[q]);
             }
         }
     }
