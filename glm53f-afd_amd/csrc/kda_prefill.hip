@@ -631,10 +631,13 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             }
         }
     }
-    __syncthreads();
-    // U^T [value][row] is now what VT holds
-    for (int e = t; e < DV * (CH / 8); e += THREADS) {
-        const int v = e >> 3, piece = e & 7;
+    // U^T [value][row] is now what VT holds. A wave copies out the 32 values of its own two tiles: its own writes,
+    // which its reads follow in order, so no barrier in between.
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = lane + 64 * j, v = 32 * wave + (e >> 3), piece = e & 7;
         *reinterpret_cast<uint4*>(wsc + WS_UT + (v * CH + 8 * piece) * 2) =
             *reinterpret_cast<const uint4*>(VT + v * LD64 + 8 * piece);
     }
