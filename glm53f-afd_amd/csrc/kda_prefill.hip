@@ -854,8 +854,8 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
             _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                        \
                 X_.q[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_QG + off_a + 4096 * ks);                         \
-            _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                        \
-                X_.m[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_M + off_a + 4096 * ks);                          \
+            X_.m[0] = *reinterpret_cast<const u32x4*>(src_ + WS_M + off_a);                                         \
+            if (wave >= 2) X_.m[1] = *reinterpret_cast<const u32x4*>(src_ + WS_M + off_a + 4096);                   \
         }
         // The read-out of a chunk starts after the chunk's second barrier, when both the state and V' are in LDS and
         // the state waves are done with their long reads of the state; the rows are stored while the state waves
@@ -889,11 +889,14 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             // four consecutive values of one row and stores them as one 8-byte piece
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) accY[nt] = zero;
+            // M is lower triangular: rows 0..31 (waves 0 and 1) have nothing in its columns 32..63, which are neither
+            // loaded nor multiplied
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
+            for (int nt = 0; nt < NT; ++nt) accY[nt] = mfma_f16(frag(Vl, LD64, SUB * nt, 0, lane), as_u4(x.m[0]), accY[nt]);
+            if (wave >= 2) {
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    accY[nt] = mfma_f16(frag(Vl, LD64, SUB * nt, 32 * ks, lane), as_u4(x.m[ks]), accY[nt]);
+                for (int nt = 0; nt < NT; ++nt) accY[nt] = mfma_f16(frag(Vl, LD64, SUB * nt, 32, lane), as_u4(x.m[1]), accY[nt]);
+            }
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
