@@ -165,8 +165,11 @@ __device__ __forceinline__ float row_sum(float (&x)[NP]) {
     }
 #pragma unroll
     for (int p = 0; p < NP; ++p) x[p] = x[p] + lane_xor16<8>(x[p]);
+    // After the step above lanes l and l ^ 8 hold the same bits, so the value of lane l ^ 4 is also what the lane four
+    // further round the row holds: one rotation, which folds into the add.
 #pragma unroll
-    for (int p = 0; p < NP; ++p) x[p] = x[p] + lane_xor16<4>(x[p]);
+    for (int p = 0; p < NP; ++p)
+        x[p] = x[p] + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x[p]), 0x124, 0xf, 0xf, true));
 #pragma unroll
     for (int p = 0; p < NP; ++p) x[p] = x[p] + lane_xor16<2>(x[p]);
 #pragma unroll
