@@ -260,8 +260,15 @@ __global__ void __launch_bounds__(THREADS, 4) chain_kernel(
             const float o = read_row<S>(s, qq);
             if (lane % M::LPR == 0) ys[row] = bfround(o);
             raw[j] = pack<S>(s);        // rounds a bf16 state (after the row's read-out)
-            if (ck_row != nullptr) st128((ck_row + j * M::RPS * DK) + soff_lane, raw[j]);
-            if (st_row != nullptr) st128((st_row + j * M::RPS * DK) + soff_lane, raw[j]);
+            if constexpr (M::kRound) {
+                // a bf16 state has registers to spare for the eight offsets: 32 bits on top of a scalar base
+                const unsigned off_j = soff_lane + (unsigned)(j * M::RPS * DK);
+                if (ck_row != nullptr) st128(ck_row + off_j, raw[j]);
+                if (st_row != nullptr) st128(st_row + off_j, raw[j]);
+            } else {
+                if (ck_row != nullptr) st128((ck_row + j * M::RPS * DK) + soff_lane, raw[j]);
+                if (st_row != nullptr) st128((st_row + j * M::RPS * DK) + soff_lane, raw[j]);
+            }
         }
         if (k_save != nullptr) {
             const long long base = (gr * H + h) * DK;
