@@ -1,0 +1,93 @@
+"""The entry points under HIP graph capture: they allocate nothing and clear nothing with memsets, so a decode
+round and a prefill call can be recorded once and replayed. Every replay is checked against the same calls made
+eagerly, bit for bit, with eager work and synchronisations between the replays.
+
+(The reference has no graph path; its engine launches eagerly on one stream. This is what a caller that captures
+its step gets from this library.)
+"""
+import numpy as np
+import pytest
+import torch
+
+from glm53f_kda import WINDOW, channels, ffi, state_len
+from oracle import kda_oracle as o
+
+import harness as hs
+from harness import ptr
+
+pytestmark = pytest.mark.gpu
+
+NO_SAVES = (None, None, None, None)
+
+
+def decode_call(p, w, pool, slots, sr, meta, stream):
+    """One decode round in place: chain and conv window advance in one launch per call."""
+    fn = ffi.glm53f_kda_chain_shift_batch_bf16state if pool.bf16 else ffi.glm53f_kda_chain_shift_batch
+    hs.check(fn(p.heads, meta.batch, ptr(meta.cu_rows), *sr.row_args(), ptr(pool.conv), ptr(meta.conv_off),
+                ptr(w.conv_w), ptr(pool.state), ptr(pool.state), ptr(meta.state_off), *w.args(), ptr(sr.out),
+                sr.out_stride, *NO_SAVES, stream), "chain_shift_batch")
+
+
+@pytest.mark.parametrize("bf16_state", [True, False])
+def test_a_captured_decode_round_replays_like_eager_rounds(bf16_state):
+    heads, slots_n, slots = 8, 5, [3, 0, 4]
+    p = o.synth_layer(heads, 1500)
+    w = hs.Weights(p)
+    reqs = [o.synth_rows(heads, 1, 1510 + i) for i in range(len(slots))]
+    sr = hs.StagedRows(hs.stack_rows(reqs))
+    pool_g, pool_e = hs.Pool(heads, slots_n, bf16_state, 1520), hs.Pool(heads, slots_n, bf16_state, 1520)
+    meta = hs.BatchMeta([1] * len(slots), [pool_g.conv_off(s) for s in slots], [pool_g.state_off(s) for s in slots])
+    sr_e = hs.StagedRows(hs.stack_rows(reqs))           # the eager rounds write their own output rows
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        decode_call(p, w, pool_g, slots, sr, meta, torch.cuda.current_stream().cuda_stream)
+    for replay in range(1, 4):
+        graph.replay()
+        # eager work between the replays, on the default stream, and a synchronisation
+        decode_call(p, w, pool_e, slots, sr_e, meta, None)
+        junk = torch.randn(1 << 16, device=hs.DEV).sum().item()
+        hs.sync()
+        assert np.isfinite(junk)
+        assert torch.equal(pool_g.state, pool_e.state), f"state after replay {replay}"
+        assert torch.equal(pool_g.conv, pool_e.conv), f"conv windows after replay {replay}"
+        assert np.array_equal(hs.bits(sr.out_np()), hs.bits(sr_e.out_np())), f"outputs of replay {replay}"
+
+
+def test_a_captured_prefill_call_replays_like_eager_calls():
+    heads, t = 4, 150
+    p = o.synth_layer(heads, 1600)
+    w = hs.Weights(p)
+    rows = o.synth_rows(heads, t, 1610)
+    n, cw = state_len(heads), WINDOW * channels(heads)
+    conv0, s0 = o.synth_conv_window(heads, 1620), o.synth_state(heads, 1620, 0.5)
+    ws_bytes = ffi.glm53f_kda_prefill_workspace_bytes(heads, 1, 128)        # two passes over the 150 rows
+    assert ws_bytes > 0
+
+    def buffers():
+        return dict(sr=hs.StagedRows(rows), conv=hs.to_bf16(conv0), state=hs.to_f32(s0),
+                    ws=torch.empty(ws_bytes // 4, dtype=torch.float32, device=hs.DEV))
+
+    def call(b, stream):
+        # the state is carried in place and the conv window advances, so every call starts where the last ended
+        hs.check(ffi.glm53f_kda_prefill(heads, t, *b["sr"].row_args(), ptr(b["conv"]), ptr(w.conv_w), ptr(b["state"]),
+                                        ptr(b["state"]), *w.args(), ptr(b["sr"].out), b["sr"].out_stride, 0, ptr(b["ws"]),
+                                        ws_bytes, stream), "prefill")
+
+    warm = buffers()
+    call(warm, None)                                    # the first call of a process sets kernel attributes
+    hs.sync()
+    g, e = buffers(), buffers()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(g, torch.cuda.current_stream().cuda_stream)
+    for replay in range(1, 4):
+        graph.replay()
+        call(e, None)
+        junk = torch.randn(1 << 16, device=hs.DEV).sum().item()
+        hs.sync()
+        assert np.isfinite(junk)
+        assert torch.equal(g["state"], e["state"]), f"state after replay {replay}"
+        assert torch.equal(g["conv"], e["conv"]), f"conv window after replay {replay}"
+        assert np.array_equal(hs.bits(g["sr"].out_np()), hs.bits(e["sr"].out_np())), f"outputs of replay {replay}"
+    assert len(g["conv"]) == cw and len(g["state"]) == n
