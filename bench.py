@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the KDA hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|mark|gemv|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|mark|gemv|copy|yardsticks]
 
 Prints ONE JSON line. The headline `value` is the decode step's state traffic in GB/s in the 16-slot decode configuration
 (16 slots x 1 token out of a 48-slot bf16 pool, 64 heads, 34 layers each with its own pool so the working set
@@ -526,12 +526,62 @@ def bench_copy(steps, warmup, stream):
     return {"bytes_read": 2 * n, "bytes_written": 2 * n, "ms": ms, "GBps": 4 * n / (ms * 1e-3) / 1e9}
 
 
+# ------------------------------------------------------------------------------------------------ yardsticks
+
+def bench_yardsticks(steps, warmup, stream):
+    """What this GPU moves for the kernels' memory traffic with no arithmetic behind it (kernels of
+    csrc/yardsticks/yardsticks.hip, built into libglm53f_yardsticks.so beside the library): a decode-shaped update in
+    place, verify-shaped checkpoint writes, and what one CU streams through plain, nontemporal and agent-scope
+    loads. The fractions the other legs report are best read against these."""
+    import ctypes as C
+    path = os.path.join(os.path.dirname(ffi.LIB_PATH), "libglm53f_yardsticks.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it first (python -c 'import __graft_entry__ as g; g.build()')")
+    y = C.CDLL(path)
+    y.glm53f_yardstick_update_in_place.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
+    y.glm53f_yardstick_checkpoints.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
+    y.glm53f_yardstick_stream_read.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
+    st = stream.cuda_stream
+    heads, slots_n, batch, layers = HEADS, 48, 16, LAYERS
+    slot_bytes = state_len(heads) * 2
+    pools = torch.zeros(layers, slots_n * slot_bytes // 2, dtype=torch.bfloat16, device=DEV)
+    perm = torch.randperm(slots_n, generator=torch.Generator().manual_seed(2))[:batch].to(torch.int32).to(DEV)
+
+    def sweep():
+        for l in range(layers):
+            check(y.glm53f_yardstick_update_in_place(ptr(pools[l]), ptr(perm), slot_bytes, heads, batch, st), "update")
+
+    ms = timed(sweep, steps, warmup, stream) / layers
+    res = {"decode_shaped_update": {"us_per_launch": ms * 1e3, "GBps": 2 * batch * slot_bytes / (ms * 1e-3) / 1e9,
+                                    "what": "16 slots x 64 heads: 32 KB read and written back in place per workgroup, "
+                                            "nontemporal, 34 pools in turn"}}
+    rows = 16
+    ckpt = torch.empty(slots_n * rows * slot_bytes // 2, dtype=torch.bfloat16, device=DEV)
+    ms = timed(lambda: check(y.glm53f_yardstick_checkpoints(ptr(pools[0]), ptr(ckpt), heads, slots_n, rows, st), "ckpt"),
+               max(2, steps // 2), max(1, warmup // 2), stream)
+    nbytes = slots_n * slot_bytes * (1 + rows)
+    res["verify_shaped_checkpoints"] = {"ms": ms, "GBps": nbytes / (ms * 1e-3) / 1e9,
+                                        "what": "48 slots x 64 heads: 32 KB read, written to 16 checkpoints each"}
+    del ckpt
+    src = pools.view(-1)[: (128 << 20) // 2]              # 128 MB: stays in the cache behind the L2 over the passes
+    sink = torch.zeros(1024, dtype=torch.int32, device=DEV)
+    per_cu = {}
+    for wgs in (16, 256):
+        for mode, name in ((0, "plain"), (1, "nontemporal"), (2, "agent_scope")):
+            per_wg = (128 << 20) // wgs
+            ms = timed(lambda: check(y.glm53f_yardstick_stream_read(ptr(src), per_wg, wgs, 4, mode, ptr(sink), st), "read"),
+                       max(2, steps // 4), 1, stream)
+            per_cu[f"{name}_{wgs}_workgroups"] = 4 * per_wg / (ms * 1e-3) / 1e9
+    res["GBps_per_CU_streaming_128bit_loads"] = per_cu
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "gemv", "copy"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "gemv", "copy", "yardsticks"], default=None)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -585,6 +635,12 @@ def main():
         if args.only == "gemv":
             line.update({"value": gv["roofline"]["achieved"], "ms_per_step": gv["kda_proj_1row"]["us"] / 1e3,
                          "roofline": gv["roofline"], "config": gv["config"]})
+    if args.only in (None, "yardsticks"):
+        ys = bench_yardsticks(args.steps, args.warmup, stream)
+        line["yardsticks"] = ys
+        if args.only == "yardsticks":
+            line.update({"value": ys["decode_shaped_update"]["GBps"], "ms_per_step": ys["decode_shaped_update"]["us_per_launch"] / 1e3,
+                         "config": {"workload": "memory traffic of the decode and verify kernels without their arithmetic"}})
     if args.only == "copy":
         cp = bench_copy(args.steps, args.warmup, stream)
         line.update({"copy": cp, "value": cp["GBps"], "ms_per_step": cp["ms"],
