@@ -369,6 +369,10 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         beta_s[t] = t < n ? bfround(fast_sigmoid(bf2f(b_raw))) : 0.0f;
     }
     __syncthreads();
+    // From here to the end of the chunk the phases are short and end in barriers, except for the operands: a wave in
+    // them goes ahead of the other workgroup's wave on its SIMD, which is most likely in a long elementwise phase
+    // and loses nothing by waiting a few instructions (1 % on the kernel).
+    __builtin_amdgcn_s_setprio(2);
     // the factors between sub-chunks, one channel per lane; e^{G_last} goes to the workspace. The row side of the
     // tiles is kept relative to its sub-chunk's first row (k e^{G_i - G_0}), so the factors that meet it carry
     // e^{G_0} of their sub-chunk (u) on top of the decay between the sub-chunks.
@@ -397,6 +401,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     }
 
     __syncthreads();                              // the factors are in place
+    __builtin_amdgcn_s_setprio(0);
 
     // ---- operands. Per element: ep = e^{G_i - G_0} and its reciprocal (G_0: the sub-chunk's first row, so that
     // fifteen rows of decay bound the exponent); e^{G_15 - G_i} is the last row's ep over the own one.
@@ -484,6 +489,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         put_M(accM, wave, wave);
     }
     __syncthreads();                              // the column operands of every sub-chunk are in place
+    __builtin_amdgcn_s_setprio(2);
     uint16_t* TT = reinterpret_cast<uint16_t*>(smem + I_TT);
     if (wave == 0) {
         // Sub-chunk 0 has no tiles left of its diagonal, so while the other waves compute theirs wave 0 does what
@@ -642,6 +648,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             *reinterpret_cast<const uint4*>(VT + v * LD64 + 8 * piece);
     }
     __syncthreads();                              // the next chunk's conv writes VT before its first barrier
+    __builtin_amdgcn_s_setprio(0);
     }
 }
 
