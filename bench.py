@@ -36,7 +36,7 @@ from glm53f_kda import DK, DV, HEADS, LAYERS, WINDOW, channels, ffi, state_len
 TRAFFIC_BYTES = {
     "decode_chain": (36_794 + 33_024) * 1024,            # per plain chain launch, 16 slots x 1 row
     "verify_chain": (167_880 + 1_585_201) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
-    "prefill_2048_rows": (152_477 + 148_542 + 148_598 + 36_866 + 65_741 + 32_912) * 1024,   # intra, inter, norm: read + written
+    "prefill_2048_rows": (152_067 + 148_534 + 148_598 + 36_866 + 65_741 + 32_912) * 1024,   # intra, inter, norm: read + written
     "mark_state_pages": (69_930 + 70_852) * 1024,
     "gemv_kda_proj_1row": (197_885 + 48) * 1024,         # per launch: the weights once, the activations, the outputs
 }
