@@ -1053,7 +1053,12 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
     if (chunks > needed) chunks = needed > 0 ? needed : 1;
     if (chunks > 65535) chunks = 65535;
     hipStream_t st = (hipStream_t)stream;
-    static bool attr_set = false;
+    // The large LDS allocation is an attribute of each device's copy of a kernel: set once per device.
+    constexpr int kMaxDevices = 64;
+    static bool attr_set_on[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    bool& attr_set = attr_set_on[dev];
     if (!attr_set) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(&intra_kernel<true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, INTRA_LDS) != hipSuccess ||
