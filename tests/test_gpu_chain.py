@@ -181,6 +181,48 @@ def test_batch_equals_per_request_bitwise(bf16_state):
         assert np.array_equal(hs.back(conv2[at:at + WINDOW * c]), pool.conv_of(slot))
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_ragged_rounds_against_the_oracle(seed):
+    """Seeded sweep: head counts that are no power of two, 0 to 17 rows per request, shuffled slots, either state
+    type, in place or to a fresh buffer, with or without the conv window advance in the same launch. The state
+    and every output row of every request against the CPU chain run on that request alone: the bf16-stored state
+    with the reference's rounding points to a bf16 step (device expf), the f32 state to 1e-3."""
+    rng = np.random.default_rng(8000 + seed)
+    heads = int(rng.choice([1, 2, 3, 5, 8]))
+    batch = int(rng.integers(1, 8))
+    lens = [int(rng.choice([0, 1, 1, 1, 2, 3, 7, 8, 16, 17])) for _ in range(batch)]
+    slots_n = batch + int(rng.integers(0, 3))
+    slots = [int(x) for x in rng.permutation(slots_n)[:batch]]
+    bf16_state, shift = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    write = "inplace" if shift else str(rng.choice(["inplace", "to"]))
+    label = f"seed {seed}: heads {heads}, lens {lens}, slots {slots} of {slots_n}, bf16 state {bf16_state}, " \
+            f"write {write}, window advance {shift}"
+    print(label, flush=True)
+    p = o.synth_layer(heads, 8100 + seed)
+    reqs = [o.synth_rows(heads, n, 8200 + 10 * seed + i) for i, n in enumerate(lens)]
+    pool = hs.Pool(heads, slots_n, bf16_state, 8300 + seed)
+    before = [(pool.conv_of(s), pool.state_of(s)) for s in range(slots_n)]
+    out, s_out, _, _, meta = hs.chain_batch_gpu(p, pool, slots, reqs, write=write, shift=shift)
+    n, cw = heads * DV, WINDOW * channels(heads)
+    run = o.chain_bf16_state if bf16_state else o.chain
+    for i, (slot, rq) in enumerate(zip(slots, reqs)):
+        conv0, s0 = before[slot]
+        got, r0, at = pool.device_state(slot, s_out), int(meta.cu_host[i]), pool.conv_off(slot)
+        want_conv = o.conv_shift(conv0, rq, rq.rows) if shift else conv0
+        assert np.array_equal(hs.back(pool.conv[at:at + cw]), want_conv), (label, i)
+        if rq.rows == 0:
+            assert np.array_equal(hs.bits(got), hs.bits(s0)), (label, i)
+            continue
+        c = run(p, conv0, s0, rq)
+        assert hs.rel_err(got, c.state) <= (2.0 ** -7 if bf16_state else 1e-3), (label, i)
+        assert hs.rel_err(out[r0 * n:(r0 + rq.rows) * n], c.out) <= 2.0 ** -7, (label, i)
+    for slot in set(range(slots_n)) - set(slots):
+        at = pool.conv_off(slot)
+        assert np.array_equal(hs.back(pool.conv[at:at + cw]), before[slot][0]), (label, slot)
+        if write == "inplace":
+            assert np.array_equal(hs.bits(pool.device_state(slot, s_out)), hs.bits(before[slot][1])), (label, slot)
+
+
 def test_bf16_state_window_equals_serial_steps_and_replays():
     """gpu_bf16_state.rs:330-417: an R-row window == R serial single-row steps bitwise (outputs, state, saves),
     verify without a state write leaves the pool untouched, the replay of every prefix == the CPU's
