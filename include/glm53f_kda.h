@@ -76,17 +76,12 @@ typedef uint16_t glm53f_bf16;
  * out           bf16 rows of [H*128] at out + r*out_stride.
  * k_save, v_save, g_save, b_save: replay inputs of rows 0..rows-1, all NULL or all set.
  */
-int glm53f_kda_chain(int32_t heads, int32_t rows,
-                     const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
-                     const glm53f_bf16* a, int64_t a_stride,
-                     const glm53f_bf16* g, int64_t g_stride,
-                     const glm53f_bf16* conv, const glm53f_bf16* conv_w,
-                     const float* state_in, float* state_out,
-                     const float* a_log, const float* dt_bias, const glm53f_bf16* norm_w,
-                     float eps, float lower,
-                     glm53f_bf16* out, int64_t out_stride,
-                     float* k_save, glm53f_bf16* v_save, float* g_save, float* b_save,
-                     glm53f_stream_t stream);
+int glm53f_kda_chain(int32_t heads, int32_t rows, const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
+    const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g, int64_t g_stride, const glm53f_bf16* conv,
+    const glm53f_bf16* conv_w, const float* state_in, float* state_out, const float* a_log,
+    const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out,
+    int64_t out_stride, float* k_save, glm53f_bf16* v_save, float* g_save, float* b_save,
+    glm53f_stream_t stream);
 
 /**
  * One layer, `batch` requests; workgroup (h, b) runs head h of request b. Replaces
@@ -98,18 +93,12 @@ int glm53f_kda_chain(int32_t heads, int32_t rows,
  * state_off  device int64 [batch]: request b's state is state_in + state_off[b], written to
  *            state_out + state_off[b]. Regions of different requests must not overlap.
  */
-int glm53f_kda_chain_batch(int32_t heads, int32_t batch, const int32_t* cu_rows,
-                           const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
-                           const glm53f_bf16* a, int64_t a_stride,
-                           const glm53f_bf16* g, int64_t g_stride,
-                           const glm53f_bf16* conv, const int64_t* conv_off,
-                           const glm53f_bf16* conv_w,
-                           const float* state_in, float* state_out, const int64_t* state_off,
-                           const float* a_log, const float* dt_bias, const glm53f_bf16* norm_w,
-                           float eps, float lower,
-                           glm53f_bf16* out, int64_t out_stride,
-                           float* k_save, glm53f_bf16* v_save, float* g_save, float* b_save,
-                           glm53f_stream_t stream);
+int glm53f_kda_chain_batch(int32_t heads, int32_t batch, const int32_t* cu_rows, const glm53f_bf16* p,
+    int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g,
+    int64_t g_stride, const glm53f_bf16* conv, const int64_t* conv_off, const glm53f_bf16* conv_w,
+    const float* state_in, float* state_out, const int64_t* state_off, const float* a_log, const float* dt_bias,
+    const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out, int64_t out_stride, float* k_save,
+    glm53f_bf16* v_save, float* g_save, float* b_save, glm53f_stream_t stream);
 
 /**
  * glm53f_kda_chain_batch with bf16 states (state_in, state_out, state_off in bf16 elements): f32
@@ -117,38 +106,29 @@ int glm53f_kda_chain_batch(int32_t heads, int32_t batch, const int32_t* cu_rows,
  * of R rows has the bits of R serial single-row calls. The decode step. Replaces
  * glm53f_kda_chain_batch_bf16state (header :118-130, kda.cu:356-371).
  */
-int glm53f_kda_chain_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,
-                                     const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
-                                     const glm53f_bf16* a, int64_t a_stride,
-                                     const glm53f_bf16* g, int64_t g_stride,
-                                     const glm53f_bf16* conv, const int64_t* conv_off,
-                                     const glm53f_bf16* conv_w,
-                                     const glm53f_bf16* state_in, glm53f_bf16* state_out,
-                                     const int64_t* state_off,
-                                     const float* a_log, const float* dt_bias,
-                                     const glm53f_bf16* norm_w, float eps, float lower,
-                                     glm53f_bf16* out, int64_t out_stride,
-                                     float* k_save, glm53f_bf16* v_save, float* g_save,
-                                     float* b_save, glm53f_stream_t stream);
+int glm53f_kda_chain_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows, const glm53f_bf16* p,
+    int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g,
+    int64_t g_stride, const glm53f_bf16* conv, const int64_t* conv_off, const glm53f_bf16* conv_w,
+    const glm53f_bf16* state_in, glm53f_bf16* state_out, const int64_t* state_off, const float* a_log,
+    const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out,
+    int64_t out_stride, float* k_save, glm53f_bf16* v_save, float* g_save, float* b_save,
+    glm53f_stream_t stream);
 
 /**
  * The state after the first `rows` >= 0 saved rows of a chain (0 copies). state_out may equal state_in.
  * Replaces glm53f_kda_replay (header :136-138, kda.cu:392-397).
  */
-int glm53f_kda_replay(int32_t heads, int32_t rows, const float* state_in, float* state_out,
-                      const float* k_save, const glm53f_bf16* v_save, const float* g_save,
-                      const float* b_save, glm53f_stream_t stream);
+int glm53f_kda_replay(int32_t heads, int32_t rows, const float* state_in, float* state_out, const float* k_save,
+    const glm53f_bf16* v_save, const float* g_save, const float* b_save, glm53f_stream_t stream);
 
 /**
  * Every layer of one request: layer l's state at state_in/state_out + l*state_stride, its saves at
  * k_save/v_save/g_save + l*kv_stride and b_save + l*b_stride. Replaces glm53f_kda_replay_layers
  * (header :144-148, kda.cu:399-405).
  */
-int glm53f_kda_replay_layers(int32_t heads, int32_t layers, int32_t rows,
-                             const float* state_in, float* state_out, int64_t state_stride,
-                             const float* k_save, const glm53f_bf16* v_save, const float* g_save,
-                             const float* b_save, int64_t kv_stride, int64_t b_stride,
-                             glm53f_stream_t stream);
+int glm53f_kda_replay_layers(int32_t heads, int32_t layers, int32_t rows, const float* state_in,
+    float* state_out, int64_t state_stride, const float* k_save, const glm53f_bf16* v_save, const float* g_save,
+    const float* b_save, int64_t kv_stride, int64_t b_stride, glm53f_stream_t stream);
 
 /**
  * Every layer of every request (the commit after a verify round): workgroup (l*H + h, b) replays keep[b]
@@ -156,45 +136,37 @@ int glm53f_kda_replay_layers(int32_t heads, int32_t layers, int32_t rows,
  * state_out + the same offset. keep: device int32 [batch], 0 <= keep[b] <= rows of b. Replaces
  * glm53f_kda_replay_batch (header :157-163, kda.cu:407-415).
  */
-int glm53f_kda_replay_batch(int32_t heads, int32_t layers, int32_t batch,
-                            const int32_t* cu_rows, const int32_t* keep,
-                            const float* state_in, float* state_out, int64_t state_stride,
-                            const int64_t* state_off,
-                            const float* k_save, const glm53f_bf16* v_save, const float* g_save,
-                            const float* b_save, int64_t kv_stride, int64_t b_stride,
-                            glm53f_stream_t stream);
+int glm53f_kda_replay_batch(int32_t heads, int32_t layers, int32_t batch, const int32_t* cu_rows,
+    const int32_t* keep, const float* state_in, float* state_out, int64_t state_stride,
+    const int64_t* state_off, const float* k_save, const glm53f_bf16* v_save, const float* g_save,
+    const float* b_save, int64_t kv_stride, int64_t b_stride, glm53f_stream_t stream);
 
 /**
  * glm53f_kda_replay_batch with bf16 states, rounded after every replayed row: keeping k rows gives the
  * bits of k serial single-row calls. Replaces glm53f_kda_replay_batch_bf16state (header :170-176,
  * kda.cu:417-427).
  */
-int glm53f_kda_replay_batch_bf16state(int32_t heads, int32_t layers, int32_t batch,
-                                      const int32_t* cu_rows, const int32_t* keep,
-                                      const glm53f_bf16* state_in, glm53f_bf16* state_out,
-                                      int64_t state_stride, const int64_t* state_off,
-                                      const float* k_save, const glm53f_bf16* v_save,
-                                      const float* g_save, const float* b_save, int64_t kv_stride,
-                                      int64_t b_stride, glm53f_stream_t stream);
+int glm53f_kda_replay_batch_bf16state(int32_t heads, int32_t layers, int32_t batch, const int32_t* cu_rows,
+    const int32_t* keep, const glm53f_bf16* state_in, glm53f_bf16* state_out, int64_t state_stride,
+    const int64_t* state_off, const float* k_save, const glm53f_bf16* v_save, const float* g_save,
+    const float* b_save, int64_t kv_stride, int64_t b_stride, glm53f_stream_t stream);
 
 /**
  * Advance a conv window past `keep` >= 0 kept rows, in place: window row j becomes row keep + j of
  * [window; new rows], new row r being [0, channels) of p + r*p_stride. Replaces glm53f_kda_conv_shift
  * (header :183-184, kda.cu:448-451).
  */
-int glm53f_kda_conv_shift(int32_t channels, int32_t keep, glm53f_bf16* conv,
-                          const glm53f_bf16* p, int64_t p_stride, glm53f_stream_t stream);
+int glm53f_kda_conv_shift(int32_t channels, int32_t keep, glm53f_bf16* conv, const glm53f_bf16* p,
+    int64_t p_stride, glm53f_stream_t stream);
 
 /**
  * glm53f_kda_conv_shift for every layer of every request: the window of (l, b) is
  * conv + l*conv_stride + conv_off[b]; its new rows start at p + l*p_layer_stride + cu_rows[b]*p_stride; it
  * keeps keep[b] rows. Replaces glm53f_kda_conv_shift_batch (header :191-195, kda.cu:453-460).
  */
-int glm53f_kda_conv_shift_batch(int32_t channels, int32_t layers, int32_t batch,
-                                const int32_t* cu_rows, const int32_t* keep,
-                                glm53f_bf16* conv, int64_t conv_stride, const int64_t* conv_off,
-                                const glm53f_bf16* p, int64_t p_layer_stride, int64_t p_stride,
-                                glm53f_stream_t stream);
+int glm53f_kda_conv_shift_batch(int32_t channels, int32_t layers, int32_t batch, const int32_t* cu_rows,
+    const int32_t* keep, glm53f_bf16* conv, int64_t conv_stride, const int64_t* conv_off, const glm53f_bf16* p,
+    int64_t p_layer_stride, int64_t p_stride, glm53f_stream_t stream);
 
 /**
  * Bytes of workspace for the prefill to run `rows_per_pass` rows of every request per pass; 0 on bad
@@ -214,16 +186,12 @@ int64_t glm53f_kda_prefill_workspace_bytes(int32_t heads, int32_t batch, int32_t
  * not depend on the workspace size or on how requests are batched. Replaces glm53f_kda_prefill
  * (header :223-232, kda_prefill.cu:700-710).
  */
-int glm53f_kda_prefill(int32_t heads, int32_t rows,
-                       const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
-                       const glm53f_bf16* a, int64_t a_stride,
-                       const glm53f_bf16* g, int64_t g_stride,
-                       glm53f_bf16* conv, const glm53f_bf16* conv_w,
-                       const float* state_in, float* state_out,
-                       const float* a_log, const float* dt_bias, const glm53f_bf16* norm_w,
-                       float eps, float lower,
-                       glm53f_bf16* out, int64_t out_stride, int32_t value_blocks,
-                       float* workspace, int64_t workspace_bytes, glm53f_stream_t stream);
+int glm53f_kda_prefill(int32_t heads, int32_t rows, const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
+    const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv,
+    const glm53f_bf16* conv_w, const float* state_in, float* state_out, const float* a_log,
+    const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out,
+    int64_t out_stride, int32_t value_blocks, float* workspace, int64_t workspace_bytes,
+    glm53f_stream_t stream);
 
 /**
  * glm53f_kda_prefill for a batch of requests with their own row ranges, states and conv windows.
@@ -231,16 +199,12 @@ int glm53f_kda_prefill(int32_t heads, int32_t rows,
  * overlap. Replaces glm53f_kda_prefill_batch (header :240-250, kda_prefill.cu:712-725).
  */
 int glm53f_kda_prefill_batch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t max_rows,
-                             const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
-                             const glm53f_bf16* a, int64_t a_stride,
-                             const glm53f_bf16* g, int64_t g_stride,
-                             glm53f_bf16* conv, const int64_t* conv_off,
-                             const glm53f_bf16* conv_w,
-                             const float* state_in, float* state_out, const int64_t* state_off,
-                             const float* a_log, const float* dt_bias, const glm53f_bf16* norm_w,
-                             float eps, float lower,
-                             glm53f_bf16* out, int64_t out_stride, int32_t value_blocks,
-                             float* workspace, int64_t workspace_bytes, glm53f_stream_t stream);
+    const glm53f_bf16* p, int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride,
+    const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv, const int64_t* conv_off,
+    const glm53f_bf16* conv_w, const float* state_in, float* state_out, const int64_t* state_off,
+    const float* a_log, const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower,
+    glm53f_bf16* out, int64_t out_stride, int32_t value_blocks, float* workspace, int64_t workspace_bytes,
+    glm53f_stream_t stream);
 
 /**
  * glm53f_kda_prefill_batch with bf16 states in the pool. The state is carried in f32 accumulators across a
@@ -248,17 +212,13 @@ int glm53f_kda_prefill_batch(int32_t heads, int32_t batch, const int32_t* cu_row
  * so the results still do not depend on the workspace size. Replaces glm53f_kda_prefill_batch_bf16state (header :260-270,
  * kda_prefill.cu:727-742).
  */
-int glm53f_kda_prefill_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,
-                                       int32_t max_rows, const glm53f_bf16* p, int64_t p_stride,
-                                       int64_t b_off, const glm53f_bf16* a, int64_t a_stride,
-                                       const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv,
-                                       const int64_t* conv_off, const glm53f_bf16* conv_w,
-                                       const glm53f_bf16* state_in, glm53f_bf16* state_out,
-                                       const int64_t* state_off, const float* a_log,
-                                       const float* dt_bias, const glm53f_bf16* norm_w, float eps,
-                                       float lower, glm53f_bf16* out, int64_t out_stride,
-                                       int32_t value_blocks, float* workspace,
-                                       int64_t workspace_bytes, glm53f_stream_t stream);
+int glm53f_kda_prefill_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t max_rows,
+    const glm53f_bf16* p, int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride,
+    const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv, const int64_t* conv_off,
+    const glm53f_bf16* conv_w, const glm53f_bf16* state_in, glm53f_bf16* state_out, const int64_t* state_off,
+    const float* a_log, const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower,
+    glm53f_bf16* out, int64_t out_stride, int32_t value_blocks, float* workspace, int64_t workspace_bytes,
+    glm53f_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Speculative verify with per-position state checkpoints. No counterpart in the reference: there a
@@ -273,29 +233,21 @@ int glm53f_kda_prefill_batch_bf16state(int32_t heads, int32_t batch, const int32
  * would have stored had the window ended at that row. The replay inputs may be NULL or all set.
  */
 int glm53f_kda_verify_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,
-                                      const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
-                                      const glm53f_bf16* a, int64_t a_stride,
-                                      const glm53f_bf16* g, int64_t g_stride,
-                                      const glm53f_bf16* conv, const int64_t* conv_off,
-                                      const glm53f_bf16* conv_w,
-                                      const glm53f_bf16* state_in, const int64_t* state_off,
-                                      const float* a_log, const float* dt_bias,
-                                      const glm53f_bf16* norm_w, float eps, float lower,
-                                      glm53f_bf16* out, int64_t out_stride,
-                                      glm53f_bf16* ckpt,
-                                      float* k_save, glm53f_bf16* v_save, float* g_save,
-                                      float* b_save, glm53f_stream_t stream);
+    const glm53f_bf16* p, int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride,
+    const glm53f_bf16* g, int64_t g_stride, const glm53f_bf16* conv, const int64_t* conv_off,
+    const glm53f_bf16* conv_w, const glm53f_bf16* state_in, const int64_t* state_off, const float* a_log,
+    const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out,
+    int64_t out_stride, glm53f_bf16* ckpt, float* k_save, glm53f_bf16* v_save, float* g_save, float* b_save,
+    glm53f_stream_t stream);
 
 /**
  * The commit by selection, every layer of every request: for keep[b] >= 1 the checkpoint of global row
  * cu_rows[b] + keep[b] - 1 of layer l (at ckpt + l*ckpt_layer_stride) is copied to
  * state + l*state_stride + state_off[b]; keep[b] == 0 leaves that state as it is. A pure copy: bit-exact.
  */
-int glm53f_kda_select_batch_bf16state(int32_t heads, int32_t layers, int32_t batch,
-                                      const int32_t* cu_rows, const int32_t* keep,
-                                      const glm53f_bf16* ckpt, int64_t ckpt_layer_stride,
-                                      glm53f_bf16* state, int64_t state_stride,
-                                      const int64_t* state_off, glm53f_stream_t stream);
+int glm53f_kda_select_batch_bf16state(int32_t heads, int32_t layers, int32_t batch, const int32_t* cu_rows,
+    const int32_t* keep, const glm53f_bf16* ckpt, int64_t ckpt_layer_stride, glm53f_bf16* state,
+    int64_t state_stride, const int64_t* state_off, glm53f_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------------
  * A decode round in one launch. No counterpart in the reference, whose engine runs the chain and then
@@ -310,26 +262,20 @@ int glm53f_kda_select_batch_bf16state(int32_t heads, int32_t layers, int32_t bat
  * Not for a verify round, whose windows must wait for the commit.
  */
 int glm53f_kda_chain_shift_batch(int32_t heads, int32_t batch, const int32_t* cu_rows, const glm53f_bf16* p,
-                                 int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride,
-                                 const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv,
-                                 const int64_t* conv_off, const glm53f_bf16* conv_w, const float* state_in,
-                                 float* state_out, const int64_t* state_off, const float* a_log,
-                                 const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower,
-                                 glm53f_bf16* out, int64_t out_stride, float* k_save, glm53f_bf16* v_save,
-                                 float* g_save, float* b_save, glm53f_stream_t stream);
+    int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g,
+    int64_t g_stride, glm53f_bf16* conv, const int64_t* conv_off, const glm53f_bf16* conv_w,
+    const float* state_in, float* state_out, const int64_t* state_off, const float* a_log, const float* dt_bias,
+    const glm53f_bf16* norm_w, float eps, float lower, glm53f_bf16* out, int64_t out_stride, float* k_save,
+    glm53f_bf16* v_save, float* g_save, float* b_save, glm53f_stream_t stream);
 
 /** glm53f_kda_chain_shift_batch with bf16 states in the pool (as glm53f_kda_chain_batch_bf16state). */
 int glm53f_kda_chain_shift_batch_bf16state(int32_t heads, int32_t batch, const int32_t* cu_rows,
-                                           const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
-                                           const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g,
-                                           int64_t g_stride, glm53f_bf16* conv, const int64_t* conv_off,
-                                           const glm53f_bf16* conv_w, const glm53f_bf16* state_in,
-                                           glm53f_bf16* state_out, const int64_t* state_off,
-                                           const float* a_log, const float* dt_bias,
-                                           const glm53f_bf16* norm_w, float eps, float lower,
-                                           glm53f_bf16* out, int64_t out_stride, float* k_save,
-                                           glm53f_bf16* v_save, float* g_save, float* b_save,
-                                           glm53f_stream_t stream);
+    const glm53f_bf16* p, int64_t p_stride, int64_t b_off, const glm53f_bf16* a, int64_t a_stride,
+    const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv, const int64_t* conv_off,
+    const glm53f_bf16* conv_w, const glm53f_bf16* state_in, glm53f_bf16* state_out, const int64_t* state_off,
+    const float* a_log, const float* dt_bias, const glm53f_bf16* norm_w, float eps, float lower,
+    glm53f_bf16* out, int64_t out_stride, float* k_save, glm53f_bf16* v_save, float* g_save, float* b_save,
+    glm53f_stream_t stream);
 
 /** The gfx architecture the kernels were compiled for ("gfx950"). */
 const char* glm53f_kda_arch(void);
