@@ -6,7 +6,7 @@ import subprocess
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HOST = os.path.join(ROOT, "glm53f-afd_amd", "host")
+HOST = os.path.join(ROOT, "tests", "host")
 EXE = os.path.join(HOST, "host_tests")
 
 
