@@ -91,3 +91,50 @@ def test_a_captured_prefill_call_replays_like_eager_calls():
         assert torch.equal(g["conv"], e["conv"]), f"conv window after replay {replay}"
         assert np.array_equal(hs.bits(g["sr"].out_np()), hs.bits(e["sr"].out_np())), f"outputs of replay {replay}"
     assert len(g["conv"]) == cw and len(g["state"]) == n
+
+
+def test_a_captured_verify_and_select_round_replays_like_eager_rounds():
+    """The speculative round as a caller would capture it: the checkpointing verify of every request's drafts, then
+    the select that commits each request's accepted prefix into the pool. The accepted lengths are device data, so
+    one recorded graph serves rounds with different outcomes: `keep` is rewritten between the replays."""
+    heads, slots_n, slots, lens = 8, 5, [3, 0, 4], [4, 1, 6]
+    keeps = [[4, 0, 3], [1, 1, 6], [0, 0, 0]]
+    p = o.synth_layer(heads, 1700)
+    w = hs.Weights(p)
+    reqs = [o.synth_rows(heads, n, 1710 + i) for i, n in enumerate(lens)]
+    n = state_len(heads)
+
+    def buffers():
+        pool = hs.Pool(heads, slots_n, True, 1720)
+        sr = hs.StagedRows(hs.stack_rows(reqs))
+        meta = hs.BatchMeta(lens, [pool.conv_off(s) for s in slots], [pool.state_off(s) for s in slots], keeps[0])
+        ck = torch.zeros(meta.total * n, dtype=torch.bfloat16, device=hs.DEV)
+        return dict(pool=pool, sr=sr, meta=meta, ck=ck)
+
+    def call(b, stream):
+        pool, sr, meta, ck = b["pool"], b["sr"], b["meta"], b["ck"]
+        hs.check(ffi.glm53f_kda_verify_batch_bf16state(
+            heads, meta.batch, ptr(meta.cu_rows), *sr.row_args(), ptr(pool.conv), ptr(meta.conv_off), ptr(w.conv_w),
+            ptr(pool.state), ptr(meta.state_off), *w.args(), ptr(sr.out), sr.out_stride, ptr(ck), *NO_SAVES, stream),
+            "verify")
+        hs.check(ffi.glm53f_kda_select_batch_bf16state(heads, 1, meta.batch, ptr(meta.cu_rows), ptr(meta.keep), ptr(ck),
+                                                       ck.numel(), ptr(pool.state), pool.state.numel(),
+                                                       ptr(meta.state_off), stream), "select")
+
+    g, e = buffers(), buffers()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(g, torch.cuda.current_stream().cuda_stream)
+    for replay, keep in enumerate(keeps, 1):
+        for b in (g, e):                                # this round's outcome, written where the graph reads it
+            b["meta"].keep.copy_(torch.tensor(keep, dtype=torch.int32))
+        graph.replay()
+        call(e, None)
+        junk = torch.randn(1 << 16, device=hs.DEV).sum().item()
+        hs.sync()
+        assert np.isfinite(junk)
+        assert torch.equal(g["pool"].state, e["pool"].state), f"pool after replay {replay}"
+        assert torch.equal(g["ck"], e["ck"]), f"checkpoints of replay {replay}"
+        assert np.array_equal(hs.bits(g["sr"].out_np()), hs.bits(e["sr"].out_np())), f"outputs of replay {replay}"
+    # the rounds did commit something: the pool has moved from where it started
+    assert not torch.equal(g["pool"].state, hs.Pool(heads, slots_n, True, 1720).state)
