@@ -189,10 +189,12 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
 // The same contract for three rows and more, where a lane's arithmetic (rows x 8 fused multiply-adds per weight
 // word pair) and its reads of the activations weigh as much as the weight stream: half a wave owns eight outputs
 // and walks the K steps in the outer loop, so that the rows' activations of a step are read from LDS once for all
-// eight (each accumulator still sees its products in the order of the model). 128 lanes per workgroup, 32 outputs;
-// taken when that still gives two workgroups per CU (64-lane workgroups for a smaller n measured slower than the
-// kernel above).
-constexpr int WIDE_THREADS = 128, WIDE_OUTS = 8;
+// eight (each accumulator still sees its products in the order of the model). 256 lanes per workgroup, 64 outputs:
+// every workgroup widens the rows' activations into its own LDS, and with 32 outputs per workgroup that staging
+// cost 5 to 10 % of the launch. Taken when that still gives every CU a workgroup (64-lane workgroups for a smaller
+// n measured slower than the kernel above).
+constexpr int WIDE_THREADS = 256, WIDE_OUTS = 8;
+constexpr int WIDE_BLOCK_OUTS = (WIDE_THREADS / 32) * WIDE_OUTS;   // 64 outputs share one staging of the activations
 
 template <int M, bool F32>
 __global__ void __launch_bounds__(WIDE_THREADS) gemv_wide_kernel(const uint16_t* __restrict__ x, long long ldx,
@@ -201,7 +203,7 @@ __global__ void __launch_bounds__(WIDE_THREADS) gemv_wide_kernel(const uint16_t*
                                                                  float* __restrict__ partials,
                                                                  unsigned* __restrict__ sync, void* __restrict__ out,
                                                                  long long ldo, long long o_gs) {
-    constexpr int BLOCK_OUTS = (WIDE_THREADS / 32) * WIDE_OUTS;
+    constexpr int BLOCK_OUTS = WIDE_BLOCK_OUTS;
     extern __shared__ __align__(16) unsigned char smem[];
     float* xs = reinterpret_cast<float*>(smem);                       // [M][kp]
     const int t = threadIdx.x, hw = t >> 5, l = t & 31;
@@ -332,11 +334,11 @@ int32_t launch_m(const uint16_t* x, long long ldx, long long x_gs, const uint16_
                  int groups, int n, int k, int ksplit, float* partials, unsigned* sync, void* out, long long ldo,
                  long long o_gs, hipStream_t stream) {
     const long long blocks8 = (long long)(n / 8) * ksplit * groups;   // workgroups with one output per half-wave
-    if (M >= 3 && blocks8 >= 4 * 512) {                                // 32 outputs per workgroup: two per CU and more
+    if (M >= 3 && blocks8 >= 4 * 512) {                                // 64 outputs per workgroup: one per CU and more
         const int kc = k / ksplit;
         int kp = LDS_BYTES / 2 / (4 * M) / STEP * STEP;
         if (kp > kc) kp = kc;
-        const dim3 grid((unsigned)((n + 31) / 32), (unsigned)ksplit, (unsigned)groups);
+        const dim3 grid((unsigned)((n + WIDE_BLOCK_OUTS - 1) / WIDE_BLOCK_OUTS), (unsigned)ksplit, (unsigned)groups);
         gemv_wide_kernel<M, F32><<<grid, WIDE_THREADS, (size_t)M * kp * 4, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, kc, kp,
                                                                                      partials, sync, out, ldo, o_gs);
         return (int32_t)hipGetLastError();
