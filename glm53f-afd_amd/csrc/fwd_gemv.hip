@@ -336,7 +336,9 @@ int32_t launch_m(const uint16_t* x, long long ldx, long long x_gs, const uint16_
     const long long blocks8 = (long long)(n / 8) * ksplit * groups;   // workgroups with one output per half-wave
     if (M >= 3 && blocks8 >= 4 * 512) {                                // 64 outputs per workgroup: one per CU and more
         const int kc = k / ksplit;
-        int kp = LDS_BYTES / 2 / (4 * M) / STEP * STEP;
+        // pieces of the K range whose activations fit 32 KiB; from five rows up 64 KiB, which halves the number of
+        // pieces and with them the waits for a piece's staging (two workgroups still fit a CU's LDS)
+        int kp = (M > 4 ? LDS_BYTES : LDS_BYTES / 2) / (4 * M) / STEP * STEP;
         if (kp > kc) kp = kc;
         const dim3 grid((unsigned)((n + WIDE_BLOCK_OUTS - 1) / WIDE_BLOCK_OUTS), (unsigned)ksplit, (unsigned)groups);
         gemv_wide_kernel<M, F32><<<grid, WIDE_THREADS, (size_t)M * kp * 4, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, kc, kp,

@@ -128,6 +128,9 @@ def test_gemv_kda_projection_shape():
     got8 = run(sc, x, w, 8, 1, False)
     got1 = run(sc, x, w, 1, 1, False)
     assert np.array_equal(got1.view(np.uint32), got8[:, :1].view(np.uint32))
+    for rows in range(2, 8):      # every row count of the eight-outputs kernel, whose K pieces depend on the count
+        part = run(sc, x, w, rows, 1, False)
+        assert np.array_equal(part.view(np.uint32), got8[:, :rows].view(np.uint32)), rows
     sample = rng.permutation(n)[:2048]
     want = model(x, w[:, sample], 8, 1, False)
     assert np.array_equal(got8[:, :, sample].view(np.uint32), want.view(np.uint32))
