@@ -134,6 +134,8 @@ def test_gemv_kda_projection_shape():
     sample = rng.permutation(n)[:2048]
     want = model(x, w[:, sample], 8, 1, False)
     assert np.array_equal(got8[:, :, sample].view(np.uint32), want.view(np.uint32))
+    got8f = run(sc, x, w, 8, 1, True)                 # f32 outputs: the same sums before the bf16 rounding
+    assert np.array_equal(got8f[:, :, sample].view(np.uint32), model(x, w[:, sample], 8, 1, True).view(np.uint32))
 
 
 def test_gemv_argument_checks():
