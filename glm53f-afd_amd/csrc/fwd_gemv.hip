@@ -165,7 +165,9 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
 
     // The last workgroup of this block of outputs to finish adds the splits in split order. Counters: one per 8
     // outputs as the caller sized them; this workgroup uses the one of its first 8.
-    __shared__ int last;
+    // (the flag lives where the activations were staged: every lane is past its last read of them at the barrier
+    // below, and the staging may fill all the LDS a launch can ask for without an attribute)
+    int& last = *reinterpret_cast<int*>(smem);
     __threadfence();
     __syncthreads();
     unsigned* counter = sync + (long long)g * (n / 8) + OUTS * blockIdx.x;
@@ -287,7 +289,7 @@ __global__ void __launch_bounds__(WIDE_THREADS) gemv_wide_kernel(const uint16_t*
     }
     if (nsplit == 1) return;
 
-    __shared__ int last;                          // as above: the last workgroup of these outputs adds the splits
+    int& last = *reinterpret_cast<int*>(smem);    // as above: the last workgroup of these outputs adds the splits
     __threadfence();
     __syncthreads();
     unsigned* counter = sync + (long long)g * (n / 8) + (BLOCK_OUTS / 8) * blockIdx.x;
