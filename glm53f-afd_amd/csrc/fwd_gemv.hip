@@ -10,6 +10,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "glm53f_fwd_gemv.h"
 
 namespace fwd_gemv {
@@ -369,6 +371,42 @@ int32_t launch(const uint16_t* x, long long ldx, long long x_gs, const uint16_t*
     }
 }
 
+// ---- the split-K scratch of glm53f_fwd_gemv_bf16_static: the partial sums of the splits, then the counters.
+// One copy per GPU, held until the process ends; every call on a GPU shares it.
+constexpr size_t kStaticPartialFloats = 262144;   // 1 MiB of f32 partial sums
+constexpr size_t kStaticCounters = 4096;          // 16 KiB of counters
+static __device__ __align__(256) unsigned char scratch[kStaticPartialFloats * 4 + kStaticCounters * 4];
+
+// The array's name is a host-side stand-in, not a device address: each GPU holds its own copy at its own address,
+// looked up once per device (with that device current) and kept.
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+unsigned char* scratch_on[kMaxDevices] = {};
+
+int scratch_of_current_device(unsigned char** ptr) {
+    int dev = -1;
+    const hipError_t rc = hipGetDevice(&dev);
+    if (rc != hipSuccess) return (int)rc;
+    if (dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_on[dev] == nullptr) {
+        void* p = nullptr;
+        const hipError_t sym = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (sym != hipSuccess) return (int)sym;
+        if (p == nullptr) return (int)hipErrorInvalidSymbol;
+        scratch_on[dev] = static_cast<unsigned char*>(p);
+    }
+    *ptr = scratch_on[dev];
+    return 0;
+}
+
+// The counters a launch is about to use start at zero whatever an earlier call left behind (a fill kernel, not a
+// memset: a caller may be recording the stream into a graph).
+__global__ void __launch_bounds__(THREADS) clear_counters_kernel(unsigned* counters, int count) {
+    const int i = blockIdx.x * THREADS + threadIdx.x;
+    if (i < count) counters[i] = 0u;
+}
+
 }  // namespace
 }  // namespace fwd_gemv
 
@@ -402,4 +440,31 @@ extern "C" int32_t glm53f_fwd_gemv_bf16(const uint16_t* x, int64_t ldx, int64_t 
                                   ldo, o_gstride, stream)
                    : launch<false>(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, partials, sync,
                                    out, ldo, o_gstride, stream);
+}
+
+// The same GEMV with the split-K scratch in the library's own per-GPU array: no allocation anywhere on the path.
+extern "C" int32_t glm53f_fwd_gemv_bf16_static(const uint16_t* x, int64_t ldx, int64_t x_gstride, const uint16_t* w,
+                                               int64_t ldw, int64_t w_gstride, int32_t groups, int32_t rows, int32_t n,
+                                               int32_t k, int32_t ksplit, void* out, int32_t out_f32, int64_t ldo,
+                                               int64_t o_gstride, ihipStream_t* stream) {
+    using namespace fwd_gemv;
+    if (groups < 1 || rows < 1 || rows > 8 || n < 8 || ksplit < 1) return kInvalid;
+    float* partials = nullptr;
+    unsigned* counters = nullptr;
+    if (ksplit > 1) {
+        // beyond the array: rejected, never truncated
+        const unsigned long long floats = (unsigned long long)groups * (unsigned long long)ksplit * rows * n;
+        const unsigned long long count = (unsigned long long)groups * (unsigned long long)(n / 8);
+        if (floats > kStaticPartialFloats || count > kStaticCounters) return kInvalid;
+        unsigned char* base = nullptr;
+        const int rc = scratch_of_current_device(&base);
+        if (rc != 0) return rc;
+        partials = reinterpret_cast<float*>(base);
+        counters = reinterpret_cast<unsigned*>(base + kStaticPartialFloats * 4);
+        clear_counters_kernel<<<(unsigned)((count + THREADS - 1) / THREADS), THREADS, 0, stream>>>(counters, (int)count);
+        const int32_t lrc = (int32_t)hipGetLastError();
+        if (lrc != 0) return lrc;
+    }
+    return glm53f_fwd_gemv_bf16(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, partials, counters,
+                                out, out_f32, ldo, o_gstride, stream);
 }

@@ -15,6 +15,7 @@ u32 = C.c_uint32
 PROTOTYPES = {
     "glm53f_fwd_gemv_bf16": (i32, [ptr, i64, i64, ptr, i64, i64, i32, i32, i32, i32, i32, ptr, ptr, ptr, i32, i64, i64, ptr]),
     "glm53f_fwd_gemv_ksplit": (i32, [i32, i32, i32]),
+    "glm53f_fwd_gemv_bf16_static": (i32, [ptr, i64, i64, ptr, i64, i64, i32, i32, i32, i32, i32, ptr, i32, i64, i64, ptr]),
     "glm53f_fwd_gather_rows": (i32, [ptr, i64, ptr, ptr, i64, i32, i64, ptr]),
     "glm53f_fwd_scatter_rows": (i32, [ptr, i64, ptr, ptr, i64, i32, i64, ptr]),
 }

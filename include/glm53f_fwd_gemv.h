@@ -43,6 +43,20 @@ int32_t glm53f_fwd_gemv_bf16(const uint16_t* x, int64_t ldx, int64_t x_gstride, 
  *  (reference: glm53f_forward.h:43-45, gemv_bf16.cu:141-152) */
 int32_t glm53f_fwd_gemv_ksplit(int32_t groups, int32_t n, int32_t k);
 
+/** glm53f_fwd_gemv_bf16 for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ *  harnesses that forbid hipMalloc): the same arguments without `partials` and `sync`, which live in an array the
+ *  library holds on every GPU it runs on (1 MiB of partial sums and 4,096 counters, until the process ends). The
+ *  same kernels, the same bits. It has no counterpart in the reference, whose callers bring their own scratch.
+ *  With ksplit > 1 the call is rejected (1) when groups * ksplit * rows * n > 262,144 partial sums or
+ *  groups * n / 8 > 4,096 counters; with ksplit == 1 the array is not touched. Calls no hipMalloc, hipFree or
+ *  other allocating routine; the first call on a device looks the array's address up (make it before a capture).
+ *  Every call on a GPU shares that GPU's array: the counters a call uses are cleared by a kernel on `stream` before
+ *  its launch, and calls that overlap on one GPU (two streams, two threads) race. */
+int32_t glm53f_fwd_gemv_bf16_static(const uint16_t* x, int64_t ldx, int64_t x_gstride, const uint16_t* w,
+                                    int64_t ldw, int64_t w_gstride, int32_t groups, int32_t rows, int32_t n,
+                                    int32_t k, int32_t ksplit, void* out, int32_t out_f32, int64_t ldo,
+                                    int64_t o_gstride, struct ihipStream_t* stream);
+
 #ifdef __cplusplus
 }
 #endif
