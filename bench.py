@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the KDA hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|mark|gemv|copy|yardsticks]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|mark|gemv|copy]
 
 Prints ONE JSON line. The headline `value` is the decode step's state traffic in GB/s in the 16-slot decode configuration
 (16 slots x 1 token out of a 48-slot bf16 pool, 64 heads, 34 layers each with its own pool so the working set
@@ -45,6 +45,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
 DEV = "cuda:0"
 
 METRIC = "KDA prefill tok/s per layer at T=8K (MFMA %); decode state GB/s at 16 slots"
+PREFILL_DTYPE = "fp16 MFMA operands, f32 accumulate"
 
 
 def ptr(t, off=0):
@@ -147,9 +148,8 @@ def bench_decode(steps, warmup, stream, cpu=True):
 
     # Argument lists are built once: the timed loops only make the C calls.
     chain_fn, shift_fn = ffi.glm53f_kda_chain_batch_bf16state, ffi.glm53f_kda_conv_shift_batch
-    same = int(os.environ.get("KDA_BENCH_SAME_POOL", "0"))   # diagnostic: every layer on one pool (cache-resident)
-    chain_args = [(heads, batch, ptr(cu), *rows.row_args(), ptr(convs[0 if same else l]), ptr(coff),
-                   ptr(layer.conv_w), ptr(pools[0 if same else l]), ptr(pools[0 if same else l]), ptr(soff),
+    chain_args = [(heads, batch, ptr(cu), *rows.row_args(), ptr(convs[l]), ptr(coff),
+                   ptr(layer.conv_w), ptr(pools[l]), ptr(pools[l]), ptr(soff),
                    *layer.args(), *rows.out_args(), None, None, None, None, st) for l in range(layers)]
     shift_args = [(c, 1, batch, ptr(cu), ptr(keep), ptr(convs[l]), 0, ptr(coff), ptr(rows.p), 0, rows.p_stride, st)
                   for l in range(layers)]
@@ -215,20 +215,27 @@ def bench_decode(steps, warmup, stream, cpu=True):
         conv0 = convs[0].float().cpu().numpy()
         slots = perm.tolist()
 
-        def one_layer_step():
+        def one_layer_step(nthreads):
             for i, s in enumerate(slots):
-                o.chain_bf16_state(p, conv0[s * cw:(s + 1) * cw], pool0[s * n:(s + 1) * n], reqs[i], threads=threads)
+                o.chain_bf16_state(p, conv0[s * cw:(s + 1) * cw], pool0[s * n:(s + 1) * n], reqs[i], threads=nthreads)
 
-        one_layer_step()
-        t0, reps = time.perf_counter(), 0
-        while time.perf_counter() - t0 < 2.0:
-            one_layer_step()
-            reps += 1
-        dt = (time.perf_counter() - t0) / reps
+        def seconds_per_step(nthreads, budget):
+            one_layer_step(nthreads)
+            t0, reps = time.perf_counter(), 0
+            while reps < 1 or time.perf_counter() - t0 < budget:
+                one_layer_step(nthreads)
+                reps += 1
+            return (time.perf_counter() - t0) / reps, reps
+
+        dt, reps = seconds_per_step(threads, 2.0)
+        dt1, reps1 = seconds_per_step(1, 2.0)
         res["cpu_baseline"] = {"value": state_bytes / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
                                "sample": f"config 1 in full for one layer (16 slots x 64 heads x 1 row, bf16-rounded "
                                          f"state), {reps} repetitions of the C oracle chain_bf16_state, "
-                                         f"{dt * 1e3:.2f} ms per layer-step"}
+                                         f"{dt * 1e3:.2f} ms per layer-step",
+                               "single_thread": {"value": state_bytes / dt1 / 1e9, "unit": "GB/s", "cores": 1,
+                                                 "sample": f"the same layer-step on one thread, {reps1} repetitions, "
+                                                           f"{dt1 * 1e3:.2f} ms"}}
     return res
 
 
@@ -268,6 +275,7 @@ def bench_prefill(steps, warmup, stream, cpu=True):
                      "hbm_frac": io_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
         "config": {"workload": "benchmark configuration 2: T=8192 as 4 calls of 2048 rows on one slot, H=64, chunk 64, "
                                "bf16 rows, f32 state, conv + output gate", "workspace_MB": ws_bytes / 1e6},
+        "dtype": PREFILL_DTYPE,
     }
     if cpu:
         from oracle import kda_oracle as o
@@ -284,17 +292,25 @@ def bench_prefill(steps, warmup, stream, cpu=True):
         t0 = time.perf_counter()
         o.prefill(p, conv0, s0, rq, threads=threads)
         dt_chunked = time.perf_counter() - t0
+        sample1 = 256
+        rq1 = rows.to_oracle(o, 0, sample1)
+        t0 = time.perf_counter()
+        o.literal_chain(p, conv0, s0, rq1, threads=1)
+        dt1 = time.perf_counter() - t0
         res["cpu_baseline"] = {"value": sample / dt, "unit": "tok/s per layer", "cores": threads, "kind": "port",
                                "sample": f"the first {sample}-row lane of the prompt, 64 heads, the C oracle's literal "
                                          f"recurrent chain (conv, gates, delta rule, gated norm), {dt:.2f} s wall; "
                                          f"its chunked form takes {dt_chunked:.2f} s "
-                                         f"({sample / dt_chunked:.0f} tok/s per layer)"}
+                                         f"({sample / dt_chunked:.0f} tok/s per layer)",
+                               "single_thread": {"value": sample1 / dt1, "unit": "tok/s per layer", "cores": 1,
+                                                 "sample": f"the first {sample1} rows, 64 heads, the literal chain on one "
+                                                           f"thread, {dt1:.2f} s wall"}}
     return res
 
 
 # ------------------------------------------------------------------------------------------------ verify
 
-def bench_verify(steps, warmup, stream, saves_form=True):
+def bench_verify(steps, warmup, stream, saves_form=True, cpu=True):
     """benchmark configuration 4: 48 slots x 16 draft rows, bf16 state, a checkpoint after every row, then the commit by
     selection with an accepted length per slot drawn uniformly from [0, 16]."""
     heads, slots_n, drafts, layers = HEADS, 48, 16, 2
@@ -341,6 +357,38 @@ def bench_verify(steps, warmup, stream, saves_form=True):
         "config": {"workload": "benchmark configuration 4: verify 48 slots x 16 drafts, bf16 state, per-row checkpoints; "
                                "select with keep ~ U{0..16}", "kept_slots": kept},
     }
+    res["dtype"] = "f32 arithmetic, bf16-stored state"
+    if cpu:
+        # The CPU path of the same step on a bounded sample: 4 of the 48 slots, all 16 drafts, 64 heads, the state
+        # rounded to bf16 after every row (the checkpoints are those states).
+        from oracle import kda_oracle as o
+        threads = min(16, os.cpu_count() or 1)
+        p = o.LayerParams(heads, layer.conv_w.float().cpu().numpy(), layer.a_log.cpu().numpy(),
+                          layer.dt_bias.cpu().numpy(), layer.norm_w.float().cpu().numpy())
+        sample_slots = 4
+        pool0, conv0 = pools[0].float().cpu().numpy(), convs[0].float().cpu().numpy()
+        reqs = [rows.to_oracle(o, s * drafts, drafts) for s in range(sample_slots)]
+
+        def sample(nthreads):
+            for s in range(sample_slots):
+                o.chain_bf16_state(p, conv0[s * cw:(s + 1) * cw], pool0[s * n:(s + 1) * n], reqs[s], threads=nthreads)
+
+        def seconds(nthreads):
+            sample(nthreads)
+            t0, reps = time.perf_counter(), 0
+            while reps < 1 or time.perf_counter() - t0 < 2.0:
+                sample(nthreads)
+                reps += 1
+            return (time.perf_counter() - t0) / reps
+
+        sbytes_cpu = vbytes * sample_slots / slots_n
+        dt, dt1 = seconds(threads), seconds(1)
+        res["cpu_baseline"] = {"value": sbytes_cpu / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                               "sample": f"{sample_slots} of the 48 slots x 16 drafts x 64 heads, the C oracle's "
+                                         f"chain_bf16_state, counted with the verify pass's bytes for those slots "
+                                         f"({sbytes_cpu / 1e6:.0f} MB), {dt * 1e3:.1f} ms",
+                               "single_thread": {"value": sbytes_cpu / dt1 / 1e9, "unit": "GB/s", "cores": 1,
+                                                 "sample": f"the same sample on one thread, {dt1 * 1e3:.1f} ms"}}
     if not saves_form:
         return res
 
@@ -526,62 +574,12 @@ def bench_copy(steps, warmup, stream):
     return {"bytes_read": 2 * n, "bytes_written": 2 * n, "ms": ms, "GBps": 4 * n / (ms * 1e-3) / 1e9}
 
 
-# ------------------------------------------------------------------------------------------------ yardsticks
-
-def bench_yardsticks(steps, warmup, stream):
-    """What this GPU moves for the kernels' memory traffic with no arithmetic behind it (kernels of
-    csrc/yardsticks/yardsticks.hip, built into libglm53f_yardsticks.so beside the library): a decode-shaped update in
-    place, verify-shaped checkpoint writes, and what one CU streams through plain, nontemporal and agent-scope
-    loads. The fractions the other legs report are best read against these."""
-    import ctypes as C
-    path = os.path.join(os.path.dirname(ffi.LIB_PATH), "libglm53f_yardsticks.so")
-    if not os.path.exists(path):
-        raise RuntimeError(f"{path} is missing: build it first (python -c 'import __graft_entry__ as g; g.build()')")
-    y = C.CDLL(path)
-    y.glm53f_yardstick_update_in_place.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
-    y.glm53f_yardstick_checkpoints.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
-    y.glm53f_yardstick_stream_read.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
-    st = stream.cuda_stream
-    heads, slots_n, batch, layers = HEADS, 48, 16, LAYERS
-    slot_bytes = state_len(heads) * 2
-    pools = torch.zeros(layers, slots_n * slot_bytes // 2, dtype=torch.bfloat16, device=DEV)
-    perm = torch.randperm(slots_n, generator=torch.Generator().manual_seed(2))[:batch].to(torch.int32).to(DEV)
-
-    def sweep():
-        for l in range(layers):
-            check(y.glm53f_yardstick_update_in_place(ptr(pools[l]), ptr(perm), slot_bytes, heads, batch, st), "update")
-
-    ms = timed(sweep, steps, warmup, stream) / layers
-    res = {"decode_shaped_update": {"us_per_launch": ms * 1e3, "GBps": 2 * batch * slot_bytes / (ms * 1e-3) / 1e9,
-                                    "what": "16 slots x 64 heads: 32 KB read and written back in place per workgroup, "
-                                            "nontemporal, 34 pools in turn"}}
-    rows = 16
-    ckpt = torch.empty(slots_n * rows * slot_bytes // 2, dtype=torch.bfloat16, device=DEV)
-    ms = timed(lambda: check(y.glm53f_yardstick_checkpoints(ptr(pools[0]), ptr(ckpt), heads, slots_n, rows, st), "ckpt"),
-               max(2, steps // 2), max(1, warmup // 2), stream)
-    nbytes = slots_n * slot_bytes * (1 + rows)
-    res["verify_shaped_checkpoints"] = {"ms": ms, "GBps": nbytes / (ms * 1e-3) / 1e9,
-                                        "what": "48 slots x 64 heads: 32 KB read, written to 16 checkpoints each"}
-    del ckpt
-    src = pools.view(-1)[: (128 << 20) // 2]              # 128 MB: stays in the cache behind the L2 over the passes
-    sink = torch.zeros(1024, dtype=torch.int32, device=DEV)
-    per_cu = {}
-    for wgs in (16, 256):
-        for mode, name in ((0, "plain"), (1, "nontemporal"), (2, "agent_scope")):
-            per_wg = (128 << 20) // wgs
-            ms = timed(lambda: check(y.glm53f_yardstick_stream_read(ptr(src), per_wg, wgs, 4, mode, ptr(sink), st), "read"),
-                       max(2, steps // 4), 1, stream)
-            per_cu[f"{name}_{wgs}_workgroups"] = 4 * per_wg / (ms * 1e-3) / 1e9
-    res["GBps_per_CU_streaming_128bit_loads"] = per_cu
-    return res
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "gemv", "copy", "yardsticks"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "gemv", "copy"], default=None)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -595,7 +593,8 @@ def main():
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream()
     line = {"metric": METRIC, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32 (decode and verify: f32 arithmetic on a bf16-stored state; the prefill leg states its own)",
             "data": "synthetic"}
     dec = None
     if args.only in (None, "decode"):
@@ -615,10 +614,11 @@ def main():
         if args.only == "prefill":
             line.update({"value": pre["tok_per_s_per_layer"], "unit": "tok/s per layer",
                          "ms_per_step": pre["ms_per_8192_tokens"], "roofline": pre["roofline"],
-                         "config": pre["config"]})
+                         "config": pre["config"], "dtype": pre["dtype"]})
     if args.only in (None, "verify"):
         # alone (--only verify) the leg runs the checkpoint form only, so that a profile of it holds one kind of launch
-        ver = bench_verify(max(2, args.steps // 4), max(1, args.warmup // 2), stream, saves_form=args.only is None)
+        ver = bench_verify(max(2, args.steps // 4), max(1, args.warmup // 2), stream, saves_form=args.only is None,
+                           cpu=not args.no_cpu)
         line["verify"] = ver
         if args.only == "verify":
             line.update({"value": ver["roofline"]["achieved"], "ms_per_step": ver["verify_ms_per_layer"],
@@ -635,12 +635,6 @@ def main():
         if args.only == "gemv":
             line.update({"value": gv["roofline"]["achieved"], "ms_per_step": gv["kda_proj_1row"]["us"] / 1e3,
                          "roofline": gv["roofline"], "config": gv["config"]})
-    if args.only in (None, "yardsticks"):
-        ys = bench_yardsticks(args.steps, args.warmup, stream)
-        line["yardsticks"] = ys
-        if args.only == "yardsticks":
-            line.update({"value": ys["decode_shaped_update"]["GBps"], "ms_per_step": ys["decode_shaped_update"]["us_per_launch"] / 1e3,
-                         "config": {"workload": "memory traffic of the decode and verify kernels without their arithmetic"}})
     if args.only == "copy":
         cp = bench_copy(args.steps, args.warmup, stream)
         line.update({"copy": cp, "value": cp["GBps"], "ms_per_step": cp["ms"],
