@@ -43,16 +43,3 @@ def test_workspace_bytes_is_a_pure_host_function():
     assert ffi.glm53f_kda_prefill_workspace_bytes(64, 1, 2048) == 32 * 74240 * 64
     assert ffi.glm53f_kda_prefill_workspace_bytes(64, 1, 1) == 74240 * 64
     assert ffi.glm53f_kda_prefill_workspace_bytes(0, 1, 16) == 0
-
-
-def test_the_bench_yardsticks_are_built_beside_the_library():
-    """bench.py's yardstick kernels live in a library of their own (no product symbol in it, none of its in the
-    product library)."""
-    import ctypes
-    path = os.path.join(os.path.dirname(ffi.LIB_PATH), "libglm53f_yardsticks.so")
-    assert os.path.exists(path), "build it: python -c 'import __graft_entry__ as g; g.build()'"
-    y = ctypes.CDLL(path)
-    for name in ("glm53f_yardstick_update_in_place", "glm53f_yardstick_checkpoints", "glm53f_yardstick_stream_read"):
-        assert hasattr(y, name), name
-        assert not hasattr(ffi.lib(), name), name
-    assert not hasattr(y, "glm53f_kda_chain")
