@@ -1,25 +1,30 @@
 // KDA chunked prefill on gfx950: the delta rule over a prompt segment in the chunked (WY/UT) form, with every
-// GEMM-shaped step on the matrix cores (v_mfma_f32_16x16x32_f16; for a few tiles v_mfma_f32_16x16x4_f32; and
-// v_mfma_f32_16x16x16_f16 against the identity as a register transpose).
+// GEMM-shaped step on the matrix cores and every operand carried at f32-class precision.
 //
 // The algebra is the reference's chunk form (crates/glm53f-kda/src/chunked.rs:67-198; kernel counterpart
 // kda_prefill.cu:95-538 with 16-row chunks on CUDA cores). Here a chunk is 64 rows in four sub-chunks of 16.
 // With G the cumulative log decay inside the chunk, per key channel:
 //   L[i][j] = beta_i sum_d k_i k_j e^{G_i - G_j} (j < i),  M[i][j] = sum_d q_i k_j e^{G_i - G_j} (j <= i),
-//   T = (I + L)^-1,  T' = T diag(beta),  W = T' (k e^G),  U = T' v,  Qg = q e^G,  Kg = k e^{G_last - G};
-//   from the state S entering the chunk: V' = U - W S,  Y = Qg S + M V',  S <- e^{G_last} S + Kg^T V'.
-// e^{G_i - G_j} is factored around a reference row so that both factors are GEMM operands:
-//   * inside a sub-chunk (diagonal 16x16 blocks) around the sub-chunk's first row; one factor reaches e^{+87}
-//     (15 rows at the -5.8 bound), beyond fp16, so these few tiles run on the f32 MFMA with f32 operands;
-//   * between sub-chunks around a row in between (the end of a sub-chunk, or the middle of the chunk), where
-//     both exponents are <= 0 and the operands are fp16 (11-bit mantissa at the bf16 MFMA rate).
-// Everything that feeds the state is fp16 or f32. Only the diagonal 16x16 blocks of T are formed (in f32);
-// W and U come from a block forward substitution on [k e^G | v] with MFMA tiles (see intra_kernel).
+//   T' = (I + L)^-1 diag(beta),  Kd = k e^G,  Qg = q e^G,  Kg = k e^{G_last - G};
+//   from the state S entering the chunk: P = V - Kd S,  V' = T' P,  Y = Qg S + M V',  S <- e^{G_last} S + Kg^T V'.
+// e^{G_i - G_j} is factored around a reference row so that both factors are GEMM operands: inside a sub-chunk
+// around its first row (one factor reaches e^{+87}), between sub-chunks around a row in between (exponents <= 0).
 //
-// Kernels per pass: intra_kernel (one workgroup per two chunks of a head and request: prologue + L, M, T, W, U, Qg,
-// Kg into the workspace), inter_kernel (one workgroup per head, value-column block, request: the state in MFMA
-// accumulators across the chunks of the pass); then, once per call, norm_kernel (gated RMSNorm in place, and the conv windows'
-// advance).
+// Precision. The tiles of L and M run on the f32 MFMA (v_mfma_f32_16x16x4_f32) with f32 operands. Everything else
+// runs on v_mfma_f32_16x16x32_f16 with each operand held as a PAIR of fp16 values, hi = fp16(x s) and
+// lo = fp16(x s - hi), s a fixed power of two per operand that puts its values well inside the fp16 range. A
+// product is three instructions (hi hi, hi lo, lo hi; lo lo is below f32 rounding), which carries 22 significant
+// bits while lo is a normal fp16 number and an absolute 2^-25 / s below that (fp16 subnormals are kept by the
+// conversions and by the matrix core). Scales: k-side operands (Kd, Kg, L) 2^14 (they are bounded by 1), q-side
+// (Qg, M) 2^17 (bounded by 128^-1/2), T and T' 2, and what carries the magnitude of the values (S, P, V') 4: those
+// must stay below 16,376 in magnitude, beyond which they become infinite where the f32 recurrence stays finite.
+//
+// Kernels per pass: intra_kernel (one workgroup per two chunks of a head and request: prologue, L, M, T', Kd, Qg,
+// Kg, V into the workspace), inter_kernel (one workgroup per head, value-column block, request: the state in MFMA
+// accumulators across the chunks of the pass); then, once per call, norm_kernel (gated RMSNorm in place, and the
+// conv windows' advance).
+
+#include <mutex>
 
 #include "kda_common.h"
 
@@ -36,19 +41,24 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // a register-friendly 128-bit piece
 
-// Workspace of one (request, head, chunk), bytes.
-// Matrices that are MFMA operands of inter_kernel are stored in panels of 32 along their contraction index
-// ([panel][row][32]), so that the 16 rows x 32 of one operand fragment are 1 KiB of consecutive bytes.
-constexpr int WS_W = 0;                   // fp16 [4 key panels][64 rows][32 keys]
-constexpr int WS_UT = 16384;              // fp16 [128 values][64 rows]
-constexpr int WS_QG = 32768;              // fp16 [4 key panels][64 rows][32 keys]
-constexpr int WS_KGT = 49152;             // fp16 [2 row panels][128 keys][32 rows]
-constexpr int WS_M = 65536;               // fp16 [2 column panels][64 rows][32 columns]
-constexpr int WS_E = 73728;               // f32 [128 keys]: e^{G_last}
-constexpr int WS_BYTES = 74240;
+// Workspace of one (request, head, chunk), bytes. An MFMA operand is two planes, hi then lo, each panelled by 32
+// along its contraction index ([panel][row][32]) so that the 16 rows x 32 of one operand fragment are 1 KiB of
+// consecutive bytes.
+constexpr int PLANE16 = 16384, PLANE8 = 8192;   // from an operand's hi plane to its lo plane
+constexpr int WS_KD = 0;                  // fp16 x 2 [4 key panels][64 rows][32 keys]: -k e^G, scale 2^14
+constexpr int WS_QG = 32768;              // fp16 x 2 [4 key panels][64 rows][32 keys]: q e^G, scale 2^17
+constexpr int WS_KGT = 65536;             // fp16 x 2 [2 row panels][128 keys][32 rows]: k e^{G_last - G}, scale 2^14
+constexpr int WS_M = 98304;               // fp16 x 2 [2 column panels][64 rows][32 columns]: M, scale 2^17
+constexpr int WS_TP = 114688;             // fp16 x 2 [2 column panels][64 rows][32 columns]: T', scale 2
+constexpr int WS_VT = 131072;             // bf16 [128 values][64 rows]: v, exact
+constexpr int WS_E = 147456;              // f32 [128 keys]: e^{G_last}
+constexpr int WS_BYTES = 147968;
+constexpr float SC_K = 16384.0f;          // Kd, Kg, L
+constexpr float SC_Q = 131072.0f;         // Qg, M
+constexpr float SC_T = 2.0f;              // T, T', and the solve's right-hand sides
+constexpr float SC_V = 4.0f;              // S, P, V'
 // Element index of (row, k) in a panelled matrix with `rows` rows.
 __device__ __forceinline__ int panel_index(int rows, int row, int k) { return ((k >> 5) * rows + row) * 32 + (k & 31); }
-
 // LDS row strides in 16-bit elements: 128- and 64-wide operand rows padded by 16 bytes, so that the sixteen
 // rows one MFMA fragment read touches fall into distinct banks.
 constexpr int LD128 = 136, LD64 = 72;
@@ -71,26 +81,31 @@ __device__ __forceinline__ f32x4 mfma_f16(uint4 a, uint4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
-// LDS map of intra_kernel, bytes. 78.5 KB: two workgroups share a CU.
+// LDS map of intra_kernel, bytes. 76.5 KB: two workgroups share a CU.
 constexpr int LDD = SUB + 4;                      // f32 row stride of a diagonal block of L (16-byte multiple)
 constexpr int LDT = 40, LDZ = 24;                 // 16-bit row strides of TT and Z (16-byte multiples)
+constexpr int LDK = DK + 4;                       // f32 row stride of the column operands
 constexpr int NFAC = 14;                          // per-channel factors between sub-chunks (see factor_index)
 constexpr int I_CW = 0;                           // u32 [q | k | v][128 channels][4 taps]: the head's conv weights
 constexpr int I_DTB = I_CW + 3 * DK * TAPS * 4;   // f32 [128]: the head's dt_bias, times -rate log2(e)
 constexpr int I_TOT = I_DTB + DK * 4;             // f32 [4][128]: log2-decay totals of the sub-chunks
 constexpr int I_BETA = I_TOT + 4 * DK * 4;        // f32 [64]
-constexpr int I_KET = I_BETA + CH * 4;            // fp16 [128 keys][LD64]: k e^G, transposed
-constexpr int I_VT = I_KET + DK * LD64 * 2;       // fp16 [128 values][LD64]: v, transposed
-constexpr int I_LN = I_VT + DV * LD64 * 2;        // fp16 [64][LD64]: -L below the block diagonal, zero elsewhere
-constexpr int I_LD = I_LN + CH * LD64 * 2;        // f32 [4][16][LDD]: the diagonal blocks of L
-constexpr int I_KCE = I_LD + 4 * SUB * LDD * 4;   // fp16 [3][16][LD128]: k e^{G_end - G} of sub-chunks 0..2, row major
-constexpr int I_Z = I_KCE;                        //   later fp16 [16 column tiles][16][LDZ]: a tile of Z on its way back
-constexpr int I_FAC = I_KCE + 3 * SUB * LD128 * 2;  // f32 [NFAC][128]
-constexpr int I_TT = I_LD;                        //   later fp16 [64][LDT]: row 16 a + i holds [T_aa diag(beta) | T_aa][i][0..32)
+constexpr int I_VT = I_BETA + CH * 4;             // bf16 [128 values][LD64]: v, transposed, until it is copied out;
+constexpr int I_LD = I_VT;                        //   then f32 [4][16][LDD]: the diagonal blocks of L
+constexpr int I_TT = I_LD + 4 * SUB * LDD * 4;    //   and fp16 x 2 [64][LDT]: row 16 a + i holds [T_aa diag(beta) | T_aa][i][0..32)
+constexpr int TT_PLANE = CH * LDT;                //   (elements from the hi plane to the lo plane)
+constexpr int I_LN = I_VT + DV * LD64 * 2;        // fp16 x 2 [64][LD64]: -L below the block diagonal, zero elsewhere
+constexpr int LN_PLANE = CH * LD64;
+constexpr int I_KCE = I_LN + 2 * CH * LD64 * 2;   // f32 [3][16][LDK]: k e^{G_end - G} of sub-chunks 0..2, row major;
+constexpr int I_RT = I_KCE;                       //   later fp16 x 2 [64 columns][LD64]: the solve's right-hand sides,
+constexpr int RT_PLANE = CH * LD64;               //   transposed,
+constexpr int I_Z = I_RT + 2 * CH * LD64 * 2;     //   and fp16 x 2 [4 column tiles][16][LDZ]: a tile of Z on its way back
+constexpr int Z_PLANE = 4 * SUB * LDZ;
+constexpr int I_FAC = I_KCE + 3 * SUB * LDK * 4;  // f32 [NFAC][128]
 constexpr int INTRA_LDS = I_FAC + NFAC * DK * 4;
 constexpr int INTRA_CPW = 2;                      // consecutive chunks of a head per intra workgroup
-static_assert(16 * SUB * LDZ * 2 <= 3 * SUB * LD128 * 2, "Z fits the region of the column operands");
-static_assert(LDT * 2 == LDD * 4, "a row of TT takes the place of the row of the diagonal block it comes from");
+static_assert(I_TT + 2 * CH * LDT * 2 <= I_LN, "the diagonal blocks and TT fit where v was");
+static_assert(I_Z + 2 * Z_PLANE * 2 <= I_FAC, "the right-hand sides and Z fit the region of the column operands");
 static_assert(2 * INTRA_LDS <= 160 * 1024, "two intra workgroups per CU");
 
 // Factors e^{sum of whole sub-chunks' log decay}, per key channel: 0..3 = e^{G before sub-chunk a};
@@ -160,20 +175,51 @@ __device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
     const f32x2 v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
 }
+// x as an fp16 pair: hi = x rounded to nearest, lo = the rounding error rounded. Two values per word, the first in
+// bits 0..15.
+__device__ __forceinline__ void split_h2(float a, float b, uint32_t& hi, uint32_t& lo) {
+    hi = pack_h2(a, b);
+    const f16x2 h = __builtin_bit_cast(f16x2, hi);
+    lo = pack_h2(a - (float)h[0], b - (float)h[1]);
+}
+__device__ __forceinline__ void split_h4(const f32x4 v, uint2& hi, uint2& lo) {
+    split_h2(v[0], v[1], hi.x, lo.x);
+    split_h2(v[2], v[3], hi.y, lo.y);
+}
+__device__ __forceinline__ void split_h8(const float (&v)[8], u32x4& hi, u32x4& lo) {
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) split_h2(v[2 * e], v[2 * e + 1], h[e], l[e]);
+    hi = u32x4{h[0], h[1], h[2], h[3]};
+    lo = u32x4{l[0], l[1], l[2], l[3]};
+}
+// a b with both operands as hi/lo pairs, added to c: the lo lo term is left out.
+__device__ __forceinline__ f32x4 mfma_hl(uint4 ah, uint4 al, uint4 bh, uint4 bl, f32x4 c) {
+    c = mfma_f16(ah, bh, c);
+    c = mfma_f16(ah, bl, c);
+    return mfma_f16(al, bh, c);
+}
+__device__ __forceinline__ f32x4 scaled(const f32x4 v, float s) { return f32x4{v[0] * s, v[1] * s, v[2] * s, v[3] * s}; }
 
-// A 16 x 16 transpose on the matrix core. Every lane gives four fp16 values of its row (lane l: row l % 16, the
+// A 16 x 16 transpose on the matrix core. Every lane gives four 16-bit values of its row (lane l: row l % 16, the
 // values at positions 4 (l / 16) .. + 3 of the row's sixteen); the product with the identity comes back in the
 // accumulator layout, in which lane l holds position l % 16 of rows 4 (l / 16) .. + 3: four consecutive rows of one
 // column, which is what a store into a [column][row] matrix wants. Exact: every sum has one nonzero term.
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ f32x4 transpose16(uint32_t v01, uint32_t v23, uint2 identity) {
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4 transpose16(uint32_t v01, uint32_t v23, uint2 identity) {       // fp16 values
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
     return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, make_uint2(v01, v23)),
                                                  __builtin_bit_cast(f16x4, identity), zero, 0, 0, 0);
 }
-__device__ __forceinline__ uint2 transpose_identity(int lane) {   // rows 4 (l / 16) .. + 3 of column l % 16 of I
+__device__ __forceinline__ f32x4 transpose16_bf(uint32_t v01, uint32_t v23, uint2 identity) {    // bf16 values
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, make_uint2(v01, v23)),
+                                                     __builtin_bit_cast(s16x4, identity), zero, 0, 0, 0);
+}
+// rows 4 (l / 16) .. + 3 of column l % 16 of the identity, whose one is the 16-bit pattern `one`
+__device__ __forceinline__ uint2 transpose_identity(int lane, uint32_t one) {
     const int n = lane & 15, k0 = 4 * (lane >> 4);
-    const uint32_t one = 0x3c00u;
     return make_uint2((k0 == n ? one : 0u) | (k0 + 1 == n ? one << 16 : 0u),
                       (k0 + 2 == n ? one : 0u) | (k0 + 3 == n ? one << 16 : 0u));
 }
@@ -181,10 +227,10 @@ __device__ __forceinline__ uint2 transpose_identity(int lane) {   // rows 4 (l /
 // Pass 1: the chunks of one head of one request, everything that does not need the state, into their workspace
 // slots. Wave w owns sub-chunk w of a chunk (rows 16 w .. 16 w + 15); in the elementwise phases lane l holds row
 // l % 16 and 32 channels of it: with g = l / 16, the four pieces of eight channels 32 p + 8 g .. + 7, p = 0..3 (the
-// four lanes of a row then read 64 consecutive bytes with every load, and write 64 with every store of Qg). That
-// is the operand layout of the matrix cores for products that contract over channels, so the tiles of L and M take
-// their row side straight from registers (the diagonal ones both sides); what contracts over rows later (k e^G, v,
-// Kg) is written transposed, 16 bits at a time.
+// four lanes of a row then read 64 consecutive bytes with every load, and write 64 with every store of Kd and Qg).
+// That is the operand layout of the matrix cores for products that contract over channels, so the tiles of L and M
+// take their row side straight from registers (the diagonal ones both sides); what contracts over rows later (v,
+// Kg) is written transposed through the matrix core.
 template <bool VEC>
 __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) intra_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
@@ -204,16 +250,14 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     float* dtb_s = reinterpret_cast<float*>(smem + I_DTB);
     float* tot = reinterpret_cast<float*>(smem + I_TOT);
     float* beta_s = reinterpret_cast<float*>(smem + I_BETA);
-    uint16_t* keT = reinterpret_cast<uint16_t*>(smem + I_KET);
     uint16_t* VT = reinterpret_cast<uint16_t*>(smem + I_VT);
     uint16_t* Ln = reinterpret_cast<uint16_t*>(smem + I_LN);
     float* Ld = reinterpret_cast<float*>(smem + I_LD);
-    uint16_t* KcE = reinterpret_cast<uint16_t*>(smem + I_KCE);
+    float* KcE = reinterpret_cast<float*>(smem + I_KCE);
     float* fac = reinterpret_cast<float*>(smem + I_FAC);
     float* first = reinterpret_cast<float*>(smem + I_KCE);          // [4][128]: until the column operands go there
 
-    // the head's conv weights and dt_bias, once (the first barrier of the chunk loop publishes them... they are
-    // read before it, so one barrier here)
+    // the head's conv weights and dt_bias, once.
     // A conv weight is stored as the bf16 pair (w, 0) for an even channel and (0, w) for an odd one: the input rows
     // hold two channels per 32-bit word, and v_dot2c_f32_bf16 of such a word with the pair is w x + acc for the one
     // channel, with no unpacking.
@@ -231,7 +275,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     __syncthreads();
 
     // Every lane's own row of q | k | v (twelve 128-bit pieces: its 32 channels of each) is requested a chunk
-    // ahead: for the first chunk here, for the others while the chunk before is in its block solve. A row past the
+    // ahead: for the first chunk here, for the others while the chunk before is in its last phases. A row past the
     // end is replaced by the last real row (it only feeds rows past the end).
     u32x4 own[12];
     auto load_own = [&](int first_row) {
@@ -251,7 +295,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // what the lane holds after a transpose16: position cl_t (of the sixteen values the four lanes of a row put in:
     // lane group cl_t / 4, its value cl_t % 4) of rows rl_t .. rl_t + 3 of the sub-chunk
     const int cl_t = lane & 15, rl_t = 4 * (lane >> 4);
-    const uint2 ident = transpose_identity(lane);
+    const uint2 ident = transpose_identity(lane, 0x3c00u);          // fp16 1.0
+    const uint2 ident_bf = transpose_identity(lane, 0x3f80u);       // bf16 1.0
     const int r0 = sub0 + c * CH;                 // the chunk's first row inside the request
     const int n = min(CH, rr.rows - r0);          // its real rows
     if (n <= 0) break;
@@ -270,9 +315,9 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // the beta logit of row t (lanes of wave 0), requested now as well: its use sits right before a barrier
     const bf16_t b_raw = P[(rr.row0 + r0 + min((int)(t & (CH - 1)), n - 1)) * p_stride + b_off + h];
 
-    // ---- conv + SiLU with one bf16 rounding (q, k stay in registers; v goes to VT as fp16, exact but for values
-    // below 2^-14), and the sums of squares for the L2 norms. Rows past the request's end are not masked: their
-    // beta is zero, which removes them from L, W, U and the state update, and their outputs are never stored.
+    // ---- conv + SiLU with one bf16 rounding (q, k stay in registers; v goes to VT as it is, bf16), and the sums of
+    // squares for the L2 norms. Rows past the request's end are not masked: their beta is zero, which removes them
+    // from L, T' and the state update, and their outputs are never stored.
     uint32_t qr[16], kr[16];                      // bf16 pairs: the conv outputs are bf16 values
     float ssq = 0.0f, ssk = 0.0f;
     {
@@ -291,7 +336,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 for (int it = 0; it < 12; ++it) halo[it] = load8<VEC>(hsrc + (long long)(it >> 2) * H * DK + 32 * (it & 3));
             }
         }
-        uint32_t vh[2];
+        uint32_t vb2[2];
 #pragma unroll
         for (int it = 0; it < 12; ++it) {
             const int seg = it >> 2, p = it & 3;
@@ -317,23 +362,24 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 if (seg == 0) { qr[4 * p + d] = pair; ssq = dot2_bf16(pair, pair, ssq); }
                 if (seg == 1) { kr[4 * p + d] = pair; ssk = dot2_bf16(pair, pair, ssk); }
                 if (seg == 2) {
-                    // v as fp16, transposed into VT four rows at a time: two words are four values of the row
-                    vh[d & 1] = pack_h2(__uint_as_float(pair << 16), __uint_as_float(pair & 0xffff0000u));
+                    // v, transposed into VT four rows at a time: two words are four values of the row
+                    vb2[d & 1] = pair;
                     if (d & 1) {
-                        const f32x4 x = transpose16(vh[0], vh[1], ident);
+                        const f32x4 x = transpose16_bf(vb2[0], vb2[1], ident_bf);
                         *reinterpret_cast<uint2*>(VT + (32 * p + 8 * (cl_t >> 2) + 4 * (d >> 1) + (cl_t & 3)) * LD64 +
-                                                  SUB * wave + rl_t) = make_uint2(pack_h2(x[0], x[1]), pack_h2(x[2], x[3]));
+                                                  SUB * wave + rl_t) = make_uint2(f2bf2(x[0], x[1]), f2bf2(x[2], x[3]));
                     }
                 }
             }
         }
     }
-    // L2 norms: the four lanes of a row hold 32 channels each
+    // L2 norms: the four lanes of a row hold 32 channels each. The q side of everything below carries a factor 8
+    // (Qg and M are stored with scale 2^17 where the k side has 2^14).
     ssq += __shfl_xor(ssq, 16, 64);
     ssq += __shfl_xor(ssq, 32, 64);
     ssk += __shfl_xor(ssk, 16, 64);
     ssk += __shfl_xor(ssk, 32, 64);
-    const float qinv = __builtin_amdgcn_rsqf(ssq + 1e-6f) * 0.08838834764831845f;   // 128^-0.5
+    const float qinv = __builtin_amdgcn_rsqf(ssq + 1e-6f) * (0.08838834764831845f * (SC_Q / SC_K));   // 128^-0.5
     const float kinv = __builtin_amdgcn_rsqf(ssk + 1e-6f);
     // ---- gates: the cumulative log decay of the lane's row inside its sub-chunk, per channel
     float G[32];
@@ -371,26 +417,38 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     __syncthreads();
     // From here to the end of the chunk the phases are short and end in barriers, except for the operands: a wave in
     // them goes ahead of the other workgroup's wave on its SIMD, which is most likely in a long elementwise phase
-    // and loses nothing by waiting a few instructions (1 % on the kernel).
+    // and loses nothing by waiting a few instructions.
     __builtin_amdgcn_s_setprio(2);
+    // v leaves for the workspace ([value][row], as the inter pass adds it to its accumulators): its place in LDS
+    // is taken by the diagonal blocks after the next barrier
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int e = t + THREADS * j, v = e >> 2, piece = e & 3;       // 128 values x 4 pieces of 16 rows
+        const uint4 lo = *reinterpret_cast<const uint4*>(VT + v * LD64 + 16 * piece);
+        const uint4 hi = *reinterpret_cast<const uint4*>(VT + v * LD64 + 16 * piece + 8);
+        uint4* dst = reinterpret_cast<uint4*>(wsc + WS_VT + (v * CH + 16 * piece) * 2);
+        dst[0] = lo;
+        dst[1] = hi;
+    }
     // the factors between sub-chunks, one channel per lane; e^{G_last} goes to the workspace. The row side of the
     // tiles is kept relative to its sub-chunk's first row (k e^{G_i - G_0}), so the factors that meet it carry
-    // e^{G_0} of their sub-chunk (u) on top of the decay between the sub-chunks.
+    // e^{G_0} of their sub-chunk (u) on top of the decay between the sub-chunks. The factors that only make stored
+    // operands (0..7) carry those operands' scale.
     {
         const int d = t & (DK - 1);
         const float t0 = tot[d], t1 = tot[DK + d], t2 = tot[2 * DK + d], t3 = tot[3 * DK + d];
         const float u0 = first[d], u1 = first[DK + d], u2 = first[2 * DK + d], u3 = first[3 * DK + d];
         if (t < DK) {
-            fac[0 * DK + d] = __builtin_amdgcn_exp2f(u0);
-            fac[1 * DK + d] = __builtin_amdgcn_exp2f(t0 + u1);
-            fac[2 * DK + d] = __builtin_amdgcn_exp2f(t0 + t1 + u2);
-            fac[3 * DK + d] = __builtin_amdgcn_exp2f(t0 + t1 + t2 + u3);
+            fac[0 * DK + d] = SC_K * __builtin_amdgcn_exp2f(u0);
+            fac[1 * DK + d] = SC_K * __builtin_amdgcn_exp2f(t0 + u1);
+            fac[2 * DK + d] = SC_K * __builtin_amdgcn_exp2f(t0 + t1 + u2);
+            fac[3 * DK + d] = SC_K * __builtin_amdgcn_exp2f(t0 + t1 + t2 + u3);
             reinterpret_cast<float*>(wsc + WS_E)[d] = __builtin_amdgcn_exp2f(t0 + t1 + t2 + t3);
-            fac[4 * DK + d] = __builtin_amdgcn_exp2f(t1 + t2 + t3);
-            fac[5 * DK + d] = __builtin_amdgcn_exp2f(t2 + t3);
+            fac[4 * DK + d] = SC_K * __builtin_amdgcn_exp2f(t1 + t2 + t3);
+            fac[5 * DK + d] = SC_K * __builtin_amdgcn_exp2f(t2 + t3);
         } else {
-            fac[6 * DK + d] = __builtin_amdgcn_exp2f(t3);
-            fac[7 * DK + d] = 1.0f;
+            fac[6 * DK + d] = SC_K * __builtin_amdgcn_exp2f(t3);
+            fac[7 * DK + d] = SC_K;
             fac[factor_index(1, 0) * DK + d] = __builtin_amdgcn_exp2f(u1);
             fac[factor_index(2, 0) * DK + d] = __builtin_amdgcn_exp2f(t1 + u2);
             fac[factor_index(2, 1) * DK + d] = __builtin_amdgcn_exp2f(u2);
@@ -400,21 +458,21 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         }
     }
 
-    __syncthreads();                              // the factors are in place
+    __syncthreads();                              // the factors are in place, v has left
     __builtin_amdgcn_s_setprio(0);
 
     // ---- operands. Per element: ep = e^{G_i - G_0} and its reciprocal (G_0: the sub-chunk's first row, so that
     // fifteen rows of decay bound the exponent); e^{G_15 - G_i} is the last row's ep over the own one.
-    // The diagonal tiles of L and M take k ep, q ep (rows) and k / ep (columns) straight from registers, four
-    // channels per f32 MFMA (one per lane group); the same k ep, q ep are the row side of the other tiles and of
-    // k e^G and Qg, times factors that carry e^{G_0}.
+    // The tiles of L and M run on the f32 matrix instruction, four channels per step (one per lane group): the
+    // diagonal ones take k ep, q ep (rows) and k / ep (columns) straight from registers; the same k ep, q ep are the
+    // row side of the other tiles and of Kd and Qg, times factors that carry e^{G_0}.
     // The tiles are computed transposed (column side first in the MFMA), so an accumulator holds columns rl..rl+3 of
-    // row cl of a tile: four consecutive elements of a row of L or M, one store.
+    // row cl of a tile: four consecutive elements of a row of L or M, one store per plane.
     const int rl = 4 * (lane >> 4), cl = lane & 15;
     uint16_t* Mg = reinterpret_cast<uint16_t*>(wsc + WS_M);
     // Store a finished tile at block (rb, cb). L = beta_i * acc: a diagonal block (strictly lower) in f32 for the
-    // inversion, a block below the diagonal negated in fp16 as an MFMA operand of the block solve. M (lower with
-    // the diagonal) goes to the workspace.
+    // inversion, a block below the diagonal negated as an fp16 pair, an MFMA operand of the block solve. M (lower
+    // with the diagonal; acc holds 8 M) goes to the workspace.
     auto put_L = [&](f32x4 acc, int rb, int cb) {
         const int gi = SUB * rb + cl, gj = SUB * cb + rl;
         const float bi = beta_s[gi];
@@ -424,20 +482,26 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             for (int r = 0; r < 4; ++r) v[r] = rl + r < cl ? bi * acc[r] : 0.0f;
             *reinterpret_cast<f32x4*>(Ld + gi * LDD + rl) = v;
             *reinterpret_cast<uint2*>(Ln + gi * LD64 + gj) = make_uint2(0u, 0u);
+            *reinterpret_cast<uint2*>(Ln + LN_PLANE + gi * LD64 + gj) = make_uint2(0u, 0u);
         } else {
-            *reinterpret_cast<uint2*>(Ln + gi * LD64 + gj) =
-                make_uint2(pack_h2(-(bi * acc[0]), -(bi * acc[1])), pack_h2(-(bi * acc[2]), -(bi * acc[3])));
+            uint2 hi, lo;
+            split_h4(scaled(acc, -SC_K * bi), hi, lo);
+            *reinterpret_cast<uint2*>(Ln + gi * LD64 + gj) = hi;
+            *reinterpret_cast<uint2*>(Ln + LN_PLANE + gi * LD64 + gj) = lo;
         }
     };
     auto put_M = [&](f32x4 acc, int rb, int cb) {
         const int gi = SUB * rb + cl, gj = SUB * cb + rl;
-        float v[4];
+        f32x4 v;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = (rb != cb || gj + r <= gi) ? acc[r] : 0.0f;
-        *reinterpret_cast<uint2*>(Mg + panel_index(CH, gi, gj)) = make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
+        for (int r = 0; r < 4; ++r) v[r] = (rb != cb || gj + r <= gi) ? acc[r] * SC_K : 0.0f;
+        uint2 hi, lo;
+        split_h4(v, hi, lo);
+        *reinterpret_cast<uint2*>(Mg + panel_index(CH, gi, gj)) = hi;
+        *reinterpret_cast<uint2*>(Mg + PLANE8 / 2 + panel_index(CH, gi, gj)) = lo;
     };
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-    float kep[32], qep[32];                       // k e^{G_i - G_0}, q e^{G_i - G_0}: the row side of every tile
+    float kep[32], qep[32];                       // k e^{G_i - G_0}, 8 q e^{G_i - G_0}: the row side of every tile
     {
         f32x4 accL = zero, accM = zero;
         uint16_t* kgT = reinterpret_cast<uint16_t*>(wsc + WS_KGT);
@@ -447,7 +511,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         for (int p = 0; p < 4; ++p) {
             const f32x4 b0 = *reinterpret_cast<const f32x4*>(eB + 32 * p), b1 = *reinterpret_cast<const f32x4*>(eB + 32 * p + 4);
             const f32x4 s0 = *reinterpret_cast<const f32x4*>(eSuf + 32 * p), s1 = *reinterpret_cast<const f32x4*>(eSuf + 32 * p + 4);
-            float qg[8], kc[8], ket[8], kgt[8];
+            float qg[8], kc[8], kd[8], kgt[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const int ch = 8 * p + e;
@@ -465,25 +529,39 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 accL = __builtin_amdgcn_mfma_f32_16x16x4f32(kcd, kep[ch], accL, 0, 0, 0);
                 accM = __builtin_amdgcn_mfma_f32_16x16x4f32(kcd, qep[ch], accM, 0, 0, 0);
                 const float fb = e < 4 ? b0[e] : b1[e - 4], fs = e < 4 ? s0[e] : s1[e - 4];
-                ket[e] = kep[ch] * fb;                          // k e^{G_i} from the chunk's start
-                qg[e] = qep[ch] * fb;
+                kd[e] = -(kep[ch] * fb);                        // -2^14 k e^{G_i} from the chunk's start
+                qg[e] = qep[ch] * fb;                           // 2^17 q e^{G_i}
                 kc[e] = kcd * last;                             // k e^{G_15 - G_i}
-                kgt[e] = kc[e] * fs;
+                kgt[e] = kc[e] * fs;                            // 2^14 k e^{G_last - G_i}
             }
-            // k e^G into LDS and Kg into the workspace, both [key][row]: transposed four rows at a time
+            // Kg into the workspace [key][row]: transposed four rows at a time, the hi and the lo plane each
 #pragma unroll
             for (int hf = 0; hf < 2; ++hf) {
                 const int key = 32 * p + 8 * (cl_t >> 2) + 4 * hf + (cl_t & 3);
-                const f32x4 x = transpose16(pack_h2(ket[4 * hf], ket[4 * hf + 1]), pack_h2(ket[4 * hf + 2], ket[4 * hf + 3]), ident);
-                *reinterpret_cast<uint2*>(keT + key * LD64 + SUB * wave + rl_t) = make_uint2(pack_h2(x[0], x[1]), pack_h2(x[2], x[3]));
-                const f32x4 y = transpose16(pack_h2(kgt[4 * hf], kgt[4 * hf + 1]), pack_h2(kgt[4 * hf + 2], kgt[4 * hf + 3]), ident);
-                *reinterpret_cast<uint2*>(kgT + panel_index(DK, key, SUB * wave + rl_t)) = make_uint2(pack_h2(y[0], y[1]), pack_h2(y[2], y[3]));
+                uint32_t h01, l01, h23, l23;
+                split_h2(kgt[4 * hf], kgt[4 * hf + 1], h01, l01);
+                split_h2(kgt[4 * hf + 2], kgt[4 * hf + 3], h23, l23);
+                const f32x4 yh = transpose16(h01, h23, ident), yl = transpose16(l01, l23, ident);
+                uint16_t* dst = kgT + panel_index(DK, key, SUB * wave + rl_t);
+                *reinterpret_cast<uint2*>(dst) = make_uint2(pack_h2(yh[0], yh[1]), pack_h2(yh[2], yh[3]));
+                *reinterpret_cast<uint2*>(dst + PLANE16 / 2) = make_uint2(pack_h2(yl[0], yl[1]), pack_h2(yl[2], yl[3]));
             }
-            *reinterpret_cast<u32x4*>(wsc + WS_QG + panel_index(CH, R, 32 * p + 8 * g) * 2) =
-                u32x4{pack_h2(qg[0], qg[1]), pack_h2(qg[2], qg[3]), pack_h2(qg[4], qg[5]), pack_h2(qg[6], qg[7])};
-            if (wave < 3)
-                *reinterpret_cast<u32x4*>(KcE + (wave * SUB + i) * LD128 + 32 * p + 8 * g) =
-                    u32x4{pack_h2(kc[0], kc[1]), pack_h2(kc[2], kc[3]), pack_h2(kc[4], kc[5]), pack_h2(kc[6], kc[7])};
+            {
+                u32x4 hi, lo;
+                split_h8(kd, hi, lo);
+                unsigned char* dst = wsc + WS_KD + panel_index(CH, R, 32 * p + 8 * g) * 2;
+                *reinterpret_cast<u32x4*>(dst) = hi;
+                *reinterpret_cast<u32x4*>(dst + PLANE16) = lo;
+                split_h8(qg, hi, lo);
+                dst = wsc + WS_QG + panel_index(CH, R, 32 * p + 8 * g) * 2;
+                *reinterpret_cast<u32x4*>(dst) = hi;
+                *reinterpret_cast<u32x4*>(dst + PLANE16) = lo;
+            }
+            if (wave < 3) {
+                float* dst = KcE + (wave * SUB + i) * LDK + 32 * p + 8 * g;
+                *reinterpret_cast<f32x4*>(dst) = f32x4{kc[0], kc[1], kc[2], kc[3]};
+                *reinterpret_cast<f32x4*>(dst + 4) = f32x4{kc[4], kc[5], kc[6], kc[7]};
+            }
         }
         put_L(accL, wave, wave);
         put_M(accM, wave, wave);
@@ -495,7 +573,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         // Sub-chunk 0 has no tiles left of its diagonal, so while the other waves compute theirs wave 0 does what
         // needs the diagonal blocks only.
         // M and -L above the block diagonal are zero: blocks (0,1), (0,2), (0,3), (1,2), (1,3), (2,3), in 128-bit
-        // pieces (two per row of a block)
+        // pieces (two per row of a block), both planes
 #pragma unroll
         for (int it = 0; it < 3; ++it) {
             const int e = lane + 64 * it, blk = e >> 5, r = (e >> 1) & 15, half = e & 1;
@@ -503,11 +581,12 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             const int cb = blk < 3 ? blk + 1 : (blk < 5 ? blk - 1 : 3);
             const u32x4 z = {0u, 0u, 0u, 0u};
             *reinterpret_cast<u32x4*>(Mg + panel_index(CH, SUB * rb + r, SUB * cb + 8 * half)) = z;
+            *reinterpret_cast<u32x4*>(Mg + PLANE8 / 2 + panel_index(CH, SUB * rb + r, SUB * cb + 8 * half)) = z;
             *reinterpret_cast<u32x4*>(Ln + (SUB * rb + r) * LD64 + SUB * cb + 8 * half) = z;
+            *reinterpret_cast<u32x4*>(Ln + LN_PLANE + (SUB * rb + r) * LD64 + SUB * cb + 8 * half) = z;
         }
         // ---- the diagonal blocks of T = (I + L)^-1 in f32 by forward substitution: lane (a, j) solves column j of
-        // block a and leaves it as fp16 operands, scaled by beta_j (T' = T diag(beta)) and plain. TT takes the place
-        // of the blocks it is computed from: every lane has its block in registers before any lane writes.
+        // block a and leaves it as fp16 pairs (scale 2), scaled by beta_j (T' = T diag(beta)) and plain.
         const int a = lane >> 4, j = lane & 15;
         const float bj = beta_s[lane];
         // the block's strictly lower triangle into registers (rows as 128-bit pieces), then the substitution
@@ -530,38 +609,36 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
             for (int i = m + 1; i < SUB; ++i) acc[i] = __builtin_fmaf(l[i][m], x[m], acc[i]);
         }
-        // the reads of Ld above are complete (their values are used) and stay ahead of the writes below
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int i = 0; i < SUB; ++i) {
-            TT[(SUB * a + i) * LDT + j] = f2h(x[i] * bj);
-            TT[(SUB * a + i) * LDT + SUB + j] = f2h(x[i]);
+            const float tp = x[i] * (bj * SC_T), tn = x[i] * SC_T;
+            const uint16_t tph = f2h(tp), tnh = f2h(tn);
+            uint16_t* row = TT + (SUB * a + i) * LDT;
+            row[j] = tph;
+            row[SUB + j] = tnh;
+            row[TT_PLANE + j] = f2h(tp - h2f(tph));
+            row[TT_PLANE + SUB + j] = f2h(tn - h2f(tnh));
         }
     } else {
-        // tiles left of the diagonal: rows of sub-chunk `wave` against the columns of sub-chunk cb. In MFMA step s
-        // lane group g supplies channels 32 s + 8 g .. + 7 on both sides (which k a lane supplies is free as long as
-        // both operands agree).
+        // tiles left of the diagonal: rows of sub-chunk `wave` against the columns of sub-chunk cb, on the f32
+        // matrix instruction. In step (s, e) lane group g supplies channel 32 s + 8 g + e on both sides (which k a
+        // lane supplies is free as long as both operands agree).
 #pragma unroll 1
         for (int cb = 0; cb < wave; ++cb) {
             const float* df = fac + factor_index(wave, cb) * DK + 8 * g;
-            const uint16_t* kcol = KcE + (cb * SUB + i) * LD128 + 8 * g;
+            const float* kcol = KcE + (cb * SUB + i) * LDK + 8 * g;
             f32x4 accL = zero, accM = zero;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 const f32x4 d0 = *reinterpret_cast<const f32x4*>(df + 32 * s), d1 = *reinterpret_cast<const f32x4*>(df + 32 * s + 4);
-                const uint4 bcol = *reinterpret_cast<const uint4*>(kcol + 32 * s);
-                float ak[8], aq[8];
+                const f32x4 c0 = *reinterpret_cast<const f32x4*>(kcol + 32 * s), c1 = *reinterpret_cast<const f32x4*>(kcol + 32 * s + 4);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float f = e < 4 ? d0[e] : d1[e - 4];
-                    ak[e] = kep[8 * s + e] * f;
-                    aq[e] = qep[8 * s + e] * f;
+                    const float col = e < 4 ? c0[e] : c1[e - 4];
+                    accL = __builtin_amdgcn_mfma_f32_16x16x4f32(col, kep[8 * s + e] * f, accL, 0, 0, 0);
+                    accM = __builtin_amdgcn_mfma_f32_16x16x4f32(col, qep[8 * s + e] * f, accM, 0, 0, 0);
                 }
-                const uint4 ka = make_uint4(pack_h2(ak[0], ak[1]), pack_h2(ak[2], ak[3]), pack_h2(ak[4], ak[5]), pack_h2(ak[6], ak[7]));
-                const uint4 qa = make_uint4(pack_h2(aq[0], aq[1]), pack_h2(aq[2], aq[3]), pack_h2(aq[4], aq[5]), pack_h2(aq[6], aq[7]));
-                accL = mfma_f16(bcol, ka, accL);
-                accM = mfma_f16(bcol, qa, accM);
             }
             put_L(accL, wave, cb);
             put_M(accM, wave, cb);
@@ -570,92 +647,82 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     __syncthreads();                              // L and TT are complete; the factors and column operands are dead
     if (c + 1 < min(chunks, c_first + INTRA_CPW)) load_own(r0 + CH);   // the next chunk's rows
 
-    // ---- W = T' (k e^G) and U = T' v without the blocks of T below the diagonal: block forward substitution on
-    // R = [k e^G | v] (64 rows, 256 columns), held transposed in LDS ([column][row]: keT then VT) and solved in
-    // place, sixteen columns per tile, four tiles per wave (two of keys, two of values: the key tiles cost a product
-    // and a store more), no barrier:
+    // ---- T' = (I + L)^-1 diag(beta) without ever forming the blocks of T below the diagonal: block forward
+    // substitution on R = I (64 rows, 64 columns), held transposed in LDS ([column][row]) and solved in place.
+    // Wave w owns the sixteen columns of block column w; no barrier:
     //   Z_a = -sum_{b<a} L_ab X_b,   X_a = T'_aa R_a + T_aa Z_a.
-    // R_a enters the last product unrounded (v is exact in fp16), so X is rounded once; Z, X_b and L are fp16.
+    // Every operand is an fp16 pair with scale 2 (L: 2^14). Blocks above the diagonal come out as the zeros they are.
     {
-        uint16_t* RT = keT;                       // [256][LD64]: VT follows keT
-        static_assert(I_VT == I_KET + DK * LD64 * 2, "R^T is keT and VT side by side");
+        uint16_t* RT = reinterpret_cast<uint16_t*>(smem + I_RT);
         uint16_t* Zs = reinterpret_cast<uint16_t*>(smem + I_Z);
-        const int rl = 4 * (lane >> 4), cl = lane & 15;
-        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-        auto pack4 = [](const f32x4 v) {
-            return make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
-        };
-        // the wave's column tiles: q = 0, 1 are key tiles 2 w + q, q = 2, 3 value tiles 8 + 2 w + q - 2
-        auto tile = [&](int q) { return q < 2 ? 2 * wave + q : 6 + 2 * wave + q; };
+        // the wave's columns of the identity (2.0 as fp16: the scale), lo plane zero: lane (column cl, rows 16 q ..)
+        {
+            const int q = lane >> 4;
+            uint32_t w[8];
+#pragma unroll
+            for (int m = 0; m < 8; ++m)
+                w[m] = (q == wave && (cl >> 1) == m) ? ((cl & 1) ? 0x40000000u : 0x4000u) : 0u;
+            uint16_t* dst = RT + (SUB * wave + cl) * LD64 + SUB * q;
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4*>(dst) = u32x4{w[0], w[1], w[2], w[3]};
+            *reinterpret_cast<u32x4*>(dst + 8) = u32x4{w[4], w[5], w[6], w[7]};
+            *reinterpret_cast<u32x4*>(dst + RT_PLANE) = z;
+            *reinterpret_cast<u32x4*>(dst + RT_PLANE + 8) = z;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        uint16_t* Tg = reinterpret_cast<uint16_t*>(wsc + WS_TP);
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-            const uint4 tt = frag(TT, LDT, SUB * a, 0, lane);
+            const uint4 tth = frag(TT, LDT, SUB * a, 0, lane), ttl = frag(TT + TT_PLANE, LDT, SUB * a, 0, lane);
             if (a > 0) {
                 // Z tile [16 rows j][16 columns c]: a lane ends with four consecutive rows of one column
-                f32x4 z[4];
-                const uint4 l0 = frag(Ln, LD64, SUB * a, 0, lane);
-#pragma unroll
-                for (int q = 0; q < 4; ++q) z[q] = mfma_f16(l0, frag(RT, LD64, SUB * tile(q), 0, lane), zero);
-                if (a == 3) {
-                    const uint4 l1 = frag(Ln, LD64, SUB * a, 32, lane);
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) z[q] = mfma_f16(l1, frag(RT, LD64, SUB * tile(q), 32, lane), z[q]);
-                }
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    *reinterpret_cast<uint2*>(Zs + (tile(q) * SUB + cl) * LDZ + rl) = pack4(z[q]);
+                f32x4 z = zero;
+                z = mfma_hl(frag(Ln, LD64, SUB * a, 0, lane), frag(Ln + LN_PLANE, LD64, SUB * a, 0, lane),
+                            frag(RT, LD64, SUB * wave, 0, lane), frag(RT + RT_PLANE, LD64, SUB * wave, 0, lane), z);
+                if (a == 3)
+                    z = mfma_hl(frag(Ln, LD64, SUB * a, 32, lane), frag(Ln + LN_PLANE, LD64, SUB * a, 32, lane),
+                                frag(RT, LD64, SUB * wave, 32, lane), frag(RT + RT_PLANE, LD64, SUB * wave, 32, lane), z);
+                uint2 hi, lo;
+                split_h4(scaled(z, 1.0f / SC_K), hi, lo);
+                *reinterpret_cast<uint2*>(Zs + (wave * SUB + cl) * LDZ + rl) = hi;
+                *reinterpret_cast<uint2*>(Zs + Z_PLANE + (wave * SUB + cl) * LDZ + rl) = lo;
             }
-            // [R_a | Z_a] of a column tile as an operand [16 columns][K = 32]: k < 16 is R_a (lanes 0..31), k >= 16
-            // is Z_a (lanes 32..63): one read at a per-lane offset, no branch
-            uint4 rz[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int ct = tile(q);
-                const int off_r = I_KET + ((SUB * ct + cl) * LD64 + SUB * a + 8 * (lane >> 4)) * 2;
-                const int off_z = I_Z + ((ct * SUB + cl) * LDZ + 8 * ((lane >> 4) - 2)) * 2;
-                rz[q] = *reinterpret_cast<const uint4*>(smem + (lane < 32 ? off_r : off_z));
-                if (a == 0) {                     // Z_0 = 0
-                    const uint32_t keep = lane < 32 ? 0xffffffffu : 0u;
-                    rz[q] = make_uint4(rz[q].x & keep, rz[q].y & keep, rz[q].z & keep, rz[q].w & keep);
-                }
+            // [R_a | Z_a] of the column tile as an operand [16 columns][K = 32]: k < 16 is R_a (lanes 0..31), k >= 16
+            // is Z_a (lanes 32..63): one read per plane at a per-lane offset, no branch
+            const int off_r = I_RT + ((SUB * wave + cl) * LD64 + SUB * a + 8 * (lane >> 4)) * 2;
+            const int off_z = I_Z + ((wave * SUB + cl) * LDZ + 8 * ((lane >> 4) - 2)) * 2;
+            uint4 rzh = *reinterpret_cast<const uint4*>(smem + (lane < 32 ? off_r : off_z));
+            uint4 rzl = *reinterpret_cast<const uint4*>(smem + (lane < 32 ? off_r + RT_PLANE * 2 : off_z + Z_PLANE * 2));
+            if (a == 0) {                         // Z_0 = 0
+                const uint32_t keep = lane < 32 ? 0xffffffffu : 0u;
+                rzh = make_uint4(rzh.x & keep, rzh.y & keep, rzh.z & keep, rzh.w & keep);
+                rzl = make_uint4(rzl.x & keep, rzl.y & keep, rzl.z & keep, rzl.w & keep);
             }
-            // key columns, both ways round: the X^T tile [16 keys][16 rows] leaves a lane four consecutive keys of one
-            // row of W [row][key] for the workspace, the X tile four consecutive rows of one key for R^T; value
-            // columns: the X tile [16 rows][16 values] only
-            f32x4 x[4], xt[2];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                x[q] = mfma_f16(tt, rz[q], zero);
-                if (q < 2) xt[q] = mfma_f16(rz[q], tt, zero);
-            }
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int ct = tile(q);
-                *reinterpret_cast<uint2*>(RT + (SUB * ct + cl) * LD64 + SUB * a + rl) = pack4(x[q]);
-                if (q < 2)
-                    *reinterpret_cast<uint2*>(wsc + WS_W + panel_index(CH, SUB * a + cl, SUB * ct + rl) * 2) = pack4(xt[q]);
-            }
+            // both ways round: the X tile [16 rows][16 columns] leaves a lane four consecutive rows of one column for
+            // R^T, the X^T tile four consecutive columns of one row of T' [row][column] for the workspace
+            const f32x4 x = mfma_hl(tth, ttl, rzh, rzl, zero);
+            const f32x4 xt = mfma_hl(rzh, rzl, tth, ttl, zero);
+            uint2 hi, lo;
+            split_h4(scaled(x, 1.0f / SC_T), hi, lo);
+            *reinterpret_cast<uint2*>(RT + (SUB * wave + cl) * LD64 + SUB * a + rl) = hi;
+            *reinterpret_cast<uint2*>(RT + RT_PLANE + (SUB * wave + cl) * LD64 + SUB * a + rl) = lo;
+            split_h4(scaled(xt, 1.0f / SC_T), hi, lo);
+            *reinterpret_cast<uint2*>(Tg + panel_index(CH, SUB * a + cl, SUB * wave + rl)) = hi;
+            *reinterpret_cast<uint2*>(Tg + PLANE8 / 2 + panel_index(CH, SUB * a + cl, SUB * wave + rl)) = lo;
         }
-    }
-    // U^T [value][row] is now what VT holds. A wave copies out the 32 values of its own two tiles: its own writes,
-    // which its reads follow in order, so no barrier in between.
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int e = lane + 64 * j, v = 32 * wave + (e >> 3), piece = e & 7;
-        *reinterpret_cast<uint4*>(wsc + WS_UT + (v * CH + 8 * piece) * 2) =
-            *reinterpret_cast<const uint4*>(VT + v * LD64 + 8 * piece);
     }
     __syncthreads();                              // the next chunk's conv writes VT before its first barrier
     __builtin_amdgcn_s_setprio(0);
     }
 }
 
-// LDS map of inter_kernel, bytes: only what the waves share.
-constexpr int N_S = 0;                            // fp16 [2][NV][LD128]: the state, transposed; even and odd chunks
-constexpr int N_V = N_S + 2 * NV * LD128 * 2;     // fp16 [NV][LD64]: V', transposed
-constexpr int INTER_LDS = N_V + NV * LD64 * 2;
+// LDS map of inter_kernel, bytes: only what the waves share, each as an fp16 pair of planes.
+constexpr int S_PLANE = NV * LD128, P_PLANE = NV * LD64;   // elements from a hi plane to its lo plane
+constexpr int N_S = 0;                            // fp16 x 2 [2][NV][LD128]: the state, transposed; even and odd chunks
+constexpr int N_P = N_S + 2 * 2 * S_PLANE * 2;    // fp16 x 2 [NV][LD64]: P, transposed
+constexpr int N_V = N_P + 2 * P_PLANE * 2;        // fp16 x 2 [NV][LD64]: V', transposed
+constexpr int INTER_LDS = N_V + 2 * P_PLANE * 2;
 
 template <typename S>
 __device__ __forceinline__ float load_state_elem4(const S* p, float (&v)[4]);
@@ -679,32 +746,35 @@ __device__ __forceinline__ void store_state_elem4(bf16_t* p, const f32x4 v) {
     *reinterpret_cast<uint2*>(p) = make_uint2(f2bf2(v[0], v[1]), f2bf2(v[2], v[3]));
 }
 
-// One chunk's operands of inter_kernel as a wave holds them: MFMA fragments straight from the workspace. The
-// workgroup has two kinds of wave. State wave w (waves 0..3) owns rows 16 w .. 16 w + 15 of the chunk for V' (W, U)
-// and keys 32 w .. 32 w + 31 of the state (Kg, e^{G_last}); read-out wave w (waves 4..7) owns rows 16 w .. 16 w + 15
-// of the chunk for Y (Qg, M). Nothing a wave loads is used by another wave, so none of it passes through LDS.
+// One chunk's operands of inter_kernel as a wave holds them: MFMA fragments straight from the workspace, hi and lo
+// plane. The workgroup has two kinds of wave. State wave w (waves 0..3) owns rows 16 w .. 16 w + 15 of the chunk
+// for P (Kd, V) and keys 32 w .. 32 w + 31 of the state (Kg, e^{G_last}); read-out wave w (waves 4..7) owns rows
+// 16 w .. 16 w + 15 of the chunk for V' (T') and Y (Qg, M). Nothing a wave loads is used by another wave, so none
+// of it passes through LDS.
 struct StateOperands {
-    u32x4 w[4];                                   // rows 16 w + l % 16, keys 32 ks + 8 (l / 16) ..
-    u32x4 k[2][2];                                // keys 32 w + 16 mt + l % 16, chunk rows 32 ks + 8 (l / 16) ..
-    uint2 u[NT];                                  // value column of (nt, l % 16), rows 16 w + 4 (l / 16) ..
+    u32x4 kd[2][4];                               // [plane] rows 16 w + l % 16, keys 32 ks + 8 (l / 16) ..
+    u32x4 k[2][2][2];                             // [plane] keys 32 w + 16 mt + l % 16, chunk rows 32 ks + 8 (l / 16) ..
+    uint2 v[NT];                                  // bf16: value column of (nt, l % 16), rows 16 w + 4 (l / 16) ..
     f32x4 e[2];                                   // keys 32 w + 16 mt + 4 (l / 16) ..
 };
 struct ReadoutOperands {
-    u32x4 q[4];                                   // rows 16 w + l % 16, keys 32 ks + 8 (l / 16) ..
-    u32x4 m[2];                                   // rows 16 w + l % 16, chunk rows 32 ks + 8 (l / 16) ..
+    u32x4 q[2][4];                                // [plane] rows 16 w + l % 16, keys 32 ks + 8 (l / 16) ..
+    u32x4 m[2][2];                                // [plane] rows 16 w + l % 16, chunk rows 32 ks + 8 (l / 16) ..
+    u32x4 t[2][2];                                // the same of T'
 };
 constexpr int INTER_THREADS = 512;
 static_assert(NT == 2, "the value-column order below pairs two tiles");
-// Row m of value tile nt (of a workgroup's transposed state and V') is value column 8 (m / 4) + 4 nt + m % 4 of the
-// block: a read-out accumulator holds rows 4 g .. 4 g + 3 of both tiles, which is then eight consecutive values of
-// one output row, one 128-bit store.
+// Row m of value tile nt (of a workgroup's transposed state, P and V') is value column 8 (m / 4) + 4 nt + m % 4 of
+// the block: a read-out accumulator holds rows 4 g .. 4 g + 3 of both tiles, which is then eight consecutive values
+// of one output row, one 128-bit store.
 __device__ __forceinline__ int value_col(int nt, int m) { return 8 * (m >> 2) + 4 * nt + (m & 3); }
 
 // Pass 2: one head's NV value columns of one request through the chunks of the pass, in order. The state
-// S[128 keys][NV] lives in the MFMA accumulators of the state waves: wave w owns keys 32 w .. 32 w + 31. Only
-// V' = U - W S and S <- e S + Kg^T V' are on the path from one chunk's state to the next; the read-out
-// Y = Qg S + M V' hangs off it, so it runs in four waves of its own beside the state waves (one of each per SIMD)
-// and the chain from chunk to chunk is two short products and two barriers.
+// S[128 keys][NV] lives in the MFMA accumulators of the state waves (wave w owns keys 32 w .. 32 w + 31), in units of
+// 2^16 S, the product of the scales of Kg and V'. Per chunk, three barriers:
+//   state waves:    S -> LDS | P = V - Kd S -> LDS |  S <- e^{G_last} S  | S += Kg^T V'
+//   read-out waves: (store the rows of the chunk before)   | V' = T' P -> LDS  | Y = Qg S + M V'
+// so the chain from one chunk's state to the next is three products, and the read-out hangs off it.
 template <typename S>
 __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) inter_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
@@ -712,7 +782,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
         bf16_t* __restrict__ out, long long out_stride, const unsigned char* __restrict__ ws) {
     extern __shared__ __align__(16) unsigned char smem[];
     // Workgroups go to the eight XCDs round robin by their linear index. The value-column blocks of one head
-    // read the same W, Qg, Kg and M, so they are spaced H apart (a multiple of 8 for the model's 64 heads):
+    // read the same Kd, Qg, Kg, M and T', so they are spaced H apart (a multiple of 8 for the model's 64 heads):
     // they run on one XCD and share its L2 instead of fetching the workspace once per block.
     const int h = blockIdx.x % H, vb = blockIdx.x / H, b = blockIdx.y;
     const RowRange rr = request_rows(cu_rows, b, rows1);
@@ -727,17 +797,17 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
     const int rl = 4 * (lane >> 4), cl = lane & 15;
 
     uint16_t* Sl2 = reinterpret_cast<uint16_t*>(smem + N_S);
+    uint16_t* Pl = reinterpret_cast<uint16_t*>(smem + N_P);
     uint16_t* Vl = reinterpret_cast<uint16_t*>(smem + N_V);
     const unsigned char* wsh = ws + ((long long)b * H + h) * chunks * (long long)WS_BYTES;
     // Per-lane byte offsets of the fragments inside a chunk's workspace.
-    const unsigned off_a = (unsigned)(((SUB * wave + cl) * 32 + 8 * (lane >> 4)) * 2);   // W, Qg, M: + 4096 ks
+    const unsigned off_a = (unsigned)(((SUB * wave + cl) * 32 + 8 * (lane >> 4)) * 2);   // Kd, Qg, M, T': + 4096 ks
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
     auto as_u4 = [](const u32x4 v) { return make_uint4(v[0], v[1], v[2], v[3]); };
-    // Both kinds of wave pass the same two barriers per chunk: after the first the state of the chunk is in LDS
-    // (and every wave is done with the V' of the chunk before), after the second its V' is.
+    constexpr float S_UNITS = SC_K * SC_V;                        // the accumulators hold S_UNITS S
 
     if (state_wave) {
-        // the state: accS[mt][nt][r] = S[key 32 w + 16 mt + rl + r][value NV vb + value_col(nt, cl)]
+        // the state: accS[mt][nt][r] = S_UNITS S[key 32 w + 16 mt + rl + r][value NV vb + value_col(nt, cl)]
         f32x4 accS[2][NT];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -745,84 +815,100 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             for (int nt = 0; nt < NT; ++nt) {
                 float v4[4];
                 load_state_elem4<S>(state_in + sbase + (long long)(NV * vb + value_col(nt, cl)) * DK + 32 * wave + SUB * mt + rl, v4);
-                accS[mt][nt] = f32x4{v4[0], v4[1], v4[2], v4[3]};
+                accS[mt][nt] = f32x4{v4[0] * S_UNITS, v4[1] * S_UNITS, v4[2] * S_UNITS, v4[3] * S_UNITS};
             }
         const unsigned off_k = (unsigned)(WS_KGT + ((32 * wave + cl) * 32 + 8 * (lane >> 4)) * 2);  // + 1024 mt + 8192 ks
-        const unsigned off_u = (unsigned)(WS_UT + ((NV * vb + value_col(0, cl)) * CH + SUB * wave + rl) * 2);   // + 512 nt
+        const unsigned off_v = (unsigned)(WS_VT + ((NV * vb + value_col(0, cl)) * CH + SUB * wave + rl) * 2);   // + 512 nt
         const unsigned off_e = (unsigned)(WS_E + (32 * wave + rl) * 4);                             // + 64 mt
         // The loads of chunk C_ into operand set X_, one group at a time (each group is requested as soon as the
         // chunk two before it has used those registers). Unconditional: past the end they repeat the last chunk.
-#define KDA_LOAD_W(X_, C_)                                                                                          \
+#define KDA_LOAD_KD(X_, C_)                                                                                         \
         {                                                                                                           \
             const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
-            _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                        \
-                X_.w[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_W + off_a + 4096 * ks);                          \
+            _Pragma("unroll") for (int pl = 0; pl < 2; ++pl)                                                        \
+                _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                    \
+                    X_.kd[pl][ks] = *reinterpret_cast<const u32x4*>(src_ + WS_KD + PLANE16 * pl + off_a + 4096 * ks); \
             _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                        \
-                X_.u[nt] = *reinterpret_cast<const uint2*>(src_ + off_u + 512 * nt);                                 \
+                X_.v[nt] = *reinterpret_cast<const uint2*>(src_ + off_v + 512 * nt);                                 \
         }
 #define KDA_LOAD_KE(X_, C_)                                                                                         \
         {                                                                                                           \
             const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
             _Pragma("unroll") for (int mt = 0; mt < 2; ++mt) {                                                      \
-                _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                    \
-                    X_.k[mt][ks] = *reinterpret_cast<const u32x4*>(src_ + off_k + 1024 * mt + 8192 * ks);            \
+                _Pragma("unroll") for (int pl = 0; pl < 2; ++pl)                                                    \
+                    _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                \
+                        X_.k[pl][mt][ks] = *reinterpret_cast<const u32x4*>(src_ + PLANE16 * pl + off_k + 1024 * mt + 8192 * ks); \
                 X_.e[mt] = *reinterpret_cast<const f32x4*>(src_ + off_e + 64 * mt);                                  \
             }                                                                                                       \
         }
         // Chunk c with the operands in x; each group of x is then requested again for chunk c + 2.
         auto chunk_step = [&](const int c, StateOperands& x) __attribute__((always_inline)) {
             const int c2 = min(c + 2, nch - 1);
-            uint16_t* Sl = Sl2 + (c & 1) * (NV * LD128);
-            // S^T (fp16) for the products of the chunk
+            uint16_t* Sl = Sl2 + (c & 1) * (2 * S_PLANE);
+            // S^T as an fp16 pair (scale 4) for the products of the chunk
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    const uint32_t s0 = (uint32_t)f2h(accS[mt][nt][0]) | ((uint32_t)f2h(accS[mt][nt][1]) << 16);
-                    const uint32_t s1 = (uint32_t)f2h(accS[mt][nt][2]) | ((uint32_t)f2h(accS[mt][nt][3]) << 16);
-                    *reinterpret_cast<uint2*>(Sl + (SUB * nt + cl) * LD128 + 32 * wave + SUB * mt + rl) = make_uint2(s0, s1);
+                    uint2 hi, lo;
+                    split_h4(scaled(accS[mt][nt], SC_V / S_UNITS), hi, lo);
+                    uint16_t* dst = Sl + (SUB * nt + cl) * LD128 + 32 * wave + SUB * mt + rl;
+                    *reinterpret_cast<uint2*>(dst) = hi;
+                    *reinterpret_cast<uint2*>(dst + S_PLANE) = lo;
                 }
             __syncthreads();
-            // V' = U - W S: wave w takes rows 16 w .. 16 w + 15
-            f32x4 accV[NT];
+            // P = V - Kd S: wave w takes rows 16 w .. 16 w + 15. The workspace holds -Kd (scale 2^14), so the
+            // accumulators start at 2^16 V and end at 2^16 P.
+            f32x4 accP[NT];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) accV[nt] = zero;
+            for (int nt = 0; nt < NT; ++nt) {
+                const uint2 u = x.v[nt];
+                accP[nt] = f32x4{__uint_as_float(u.x << 16) * (SC_K * SC_V), __uint_as_float(u.x & 0xffff0000u) * (SC_K * SC_V),
+                                 __uint_as_float(u.y << 16) * (SC_K * SC_V), __uint_as_float(u.y & 0xffff0000u) * (SC_K * SC_V)};
+            }
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
-                    accV[nt] = mfma_f16(as_u4(x.w[ks]), frag(Sl, LD128, SUB * nt, 32 * ks, lane), accV[nt]);
+                    accP[nt] = mfma_hl(as_u4(x.kd[0][ks]), as_u4(x.kd[1][ks]), frag(Sl, LD128, SUB * nt, 32 * ks, lane),
+                                       frag(Sl + S_PLANE, LD128, SUB * nt, 32 * ks, lane), accP[nt]);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const uint2 u = x.u[nt];
-                const float v0 = h2f((uint16_t)(u.x & 0xffffu)) - accV[nt][0], v1 = h2f((uint16_t)(u.x >> 16)) - accV[nt][1];
-                const float v2 = h2f((uint16_t)(u.y & 0xffffu)) - accV[nt][2], v3 = h2f((uint16_t)(u.y >> 16)) - accV[nt][3];
-                const uint32_t p0 = (uint32_t)f2h(v0) | ((uint32_t)f2h(v1) << 16);
-                const uint32_t p1 = (uint32_t)f2h(v2) | ((uint32_t)f2h(v3) << 16);
-                *reinterpret_cast<uint2*>(Vl + (SUB * nt + cl) * LD64 + SUB * wave + rl) = make_uint2(p0, p1);
+                uint2 hi, lo;
+                split_h4(scaled(accP[nt], 1.0f / SC_K), hi, lo);
+                uint16_t* dst = Pl + (SUB * nt + cl) * LD64 + SUB * wave + rl;
+                *reinterpret_cast<uint2*>(dst) = hi;
+                *reinterpret_cast<uint2*>(dst + P_PLANE) = lo;
             }
-            KDA_LOAD_W(x, c2)
+            KDA_LOAD_KD(x, c2)
             __syncthreads();
-            // S <- e^{G_last} S + Kg^T V'
-            uint4 vfrag[NT][2];
+            // while the read-out waves form V': the state's decay
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks) vfrag[nt][ks] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt) {
+            for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) accS[mt][nt][r] *= x.e[mt][r];
+            __syncthreads();
+            // S <- e^{G_last} S + Kg^T V'
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
+            for (int ks = 0; ks < 2; ++ks) {
+                uint4 vh[NT], vl[NT];
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) accS[mt][nt] = mfma_f16(as_u4(x.k[mt][ks]), vfrag[nt][ks], accS[mt][nt]);
+                for (int nt = 0; nt < NT; ++nt) {
+                    vh[nt] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
+                    vl[nt] = frag(Vl + P_PLANE, LD64, SUB * nt, 32 * ks, lane);
+                }
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+                        accS[mt][nt] = mfma_hl(as_u4(x.k[0][mt][ks]), as_u4(x.k[1][mt][ks]), vh[nt], vl[nt], accS[mt][nt]);
             }
             KDA_LOAD_KE(x, c2)
             if constexpr (sizeof(S) == 2) {
-                // a bf16 state is rounded at the end of every chunk, so the result does not depend on where passes end
+                // a bf16 state is rounded at the end of every chunk, so the result does not depend on where passes
+                // end (the power-of-two units do not change which bits are kept)
 #pragma unroll
                 for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -833,9 +919,9 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
         };
         if (nch > 0) {
             StateOperands xa, xb;                 // even and odd chunks
-            KDA_LOAD_W(xa, 0) KDA_LOAD_KE(xa, 0)
+            KDA_LOAD_KD(xa, 0) KDA_LOAD_KE(xa, 0)
             const int c1 = min(1, nch - 1);
-            KDA_LOAD_W(xb, c1) KDA_LOAD_KE(xb, c1)
+            KDA_LOAD_KD(xb, c1) KDA_LOAD_KE(xb, c1)
             // in pairs, so that the operand sets are compile-time choices; an odd last chunk follows
             int c = 0;
 #pragma unroll 1
@@ -845,37 +931,46 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             }
             if (c < nch) chunk_step(c, xa);
         }
-#undef KDA_LOAD_W
+#undef KDA_LOAD_KD
 #undef KDA_LOAD_KE
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
                 store_state_elem4(state_out + sbase + (long long)(NV * vb + value_col(nt, cl)) * DK + 32 * wave + SUB * mt + rl,
-                                  accS[mt][nt]);
+                                  scaled(accS[mt][nt], 1.0f / S_UNITS));
     } else {
         // rows of `out` that start on 16-byte boundaries take eight values per store
         const bool wide_out = ((reinterpret_cast<size_t>(out) | (size_t)(out_stride * 2)) & 15) == 0;
+        const int nks = wave >= 2 ? 2 : 1;        // T' and M are lower triangular: rows 0..31 have nothing in columns 32..63
+#define KDA_LOAD_T(X_, C_)                                                                                          \
+        {                                                                                                           \
+            const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
+            _Pragma("unroll") for (int pl = 0; pl < 2; ++pl) {                                                      \
+                X_.t[pl][0] = *reinterpret_cast<const u32x4*>(src_ + WS_TP + PLANE8 * pl + off_a);                  \
+                if (nks == 2) X_.t[pl][1] = *reinterpret_cast<const u32x4*>(src_ + WS_TP + PLANE8 * pl + off_a + 4096); \
+            }                                                                                                       \
+        }
 #define KDA_LOAD_QM(X_, C_)                                                                                         \
         {                                                                                                           \
             const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
-            _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                        \
-                X_.q[ks] = *reinterpret_cast<const u32x4*>(src_ + WS_QG + off_a + 4096 * ks);                         \
-            X_.m[0] = *reinterpret_cast<const u32x4*>(src_ + WS_M + off_a);                                         \
-            if (wave >= 2) X_.m[1] = *reinterpret_cast<const u32x4*>(src_ + WS_M + off_a + 4096);                   \
+            _Pragma("unroll") for (int pl = 0; pl < 2; ++pl) {                                                      \
+                _Pragma("unroll") for (int ks = 0; ks < 4; ++ks)                                                    \
+                    X_.q[pl][ks] = *reinterpret_cast<const u32x4*>(src_ + WS_QG + PLANE16 * pl + off_a + 4096 * ks);  \
+                X_.m[pl][0] = *reinterpret_cast<const u32x4*>(src_ + WS_M + PLANE8 * pl + off_a);                   \
+                if (nks == 2) X_.m[pl][1] = *reinterpret_cast<const u32x4*>(src_ + WS_M + PLANE8 * pl + off_a + 4096); \
+            }                                                                                                       \
         }
-        // The read-out of a chunk starts after the chunk's second barrier, when both the state and V' are in LDS and
-        // the state waves are done with their long reads of the state; the rows are stored while the state waves
-        // work between the next chunk's barriers.
         f32x4 accY[NT];
         int st_c = -1;                            // the chunk whose read-out is in accY, not yet stored
         auto store_rows = [&]() __attribute__((always_inline)) {
             const int nrows = min(CH, left - st_c * CH);
             if (SUB * wave + cl < nrows) {
-                // accY[nt][r] = y[row 16 w + cl][value NV vb + 2 rl + 4 nt + r]
+                // accY[nt][r] = 2^19 y[row 16 w + cl][value NV vb + 2 rl + 4 nt + r]
+                constexpr float inv = 1.0f / (SC_Q * SC_V);
                 bf16_t* orow = out + (rr.row0 + sub0 + st_c * CH + SUB * wave + cl) * out_stride + h * DV + NV * vb + 2 * rl;
-                const u32x4 y8 = {f2bf2(accY[0][0], accY[0][1]), f2bf2(accY[0][2], accY[0][3]),
-                                  f2bf2(accY[1][0], accY[1][1]), f2bf2(accY[1][2], accY[1][3])};
+                const u32x4 y8 = {f2bf2(accY[0][0] * inv, accY[0][1] * inv), f2bf2(accY[0][2] * inv, accY[0][3] * inv),
+                                  f2bf2(accY[1][0] * inv, accY[1][1] * inv), f2bf2(accY[1][2] * inv, accY[1][3] * inv)};
                 if (wide_out) *reinterpret_cast<u32x4*>(orow) = y8;
                 else {
 #pragma unroll
@@ -888,35 +983,54 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
         };
         auto chunk_step = [&](const int c, ReadoutOperands& x) __attribute__((always_inline)) {
             const int c2 = min(c + 2, nch - 1);
-            const uint16_t* Sl = Sl2 + (c & 1) * (NV * LD128);
-            __syncthreads();
+            const uint16_t* Sl = Sl2 + (c & 1) * (2 * S_PLANE);
+            __syncthreads();                      // the chunk's state is in LDS
             if (st_c >= 0) store_rows();
-            __syncthreads();
-            // Y^T = S^T Qg^T + V'^T M^T: the state and V' on the row side of the tiles, so that a lane ends up with
-            // four consecutive values of one row and stores them as one 8-byte piece
+            __syncthreads();                      // P is in LDS
+            // V' = T' P: wave w takes rows 16 w .. 16 w + 15 (scale 2 x 4 -> 4)
+            f32x4 accV[NT];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) accY[nt] = zero;
-            // M is lower triangular: rows 0..31 (waves 0 and 1) have nothing in its columns 32..63, which are neither
-            // loaded nor multiplied
+            for (int nt = 0; nt < NT; ++nt) {
+                accV[nt] = mfma_hl(as_u4(x.t[0][0]), as_u4(x.t[1][0]), frag(Pl, LD64, SUB * nt, 0, lane),
+                                   frag(Pl + P_PLANE, LD64, SUB * nt, 0, lane), zero);
+                if (nks == 2)
+                    accV[nt] = mfma_hl(as_u4(x.t[0][1]), as_u4(x.t[1][1]), frag(Pl, LD64, SUB * nt, 32, lane),
+                                       frag(Pl + P_PLANE, LD64, SUB * nt, 32, lane), accV[nt]);
+            }
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) accY[nt] = mfma_f16(frag(Vl, LD64, SUB * nt, 0, lane), as_u4(x.m[0]), accY[nt]);
-            if (wave >= 2) {
+            for (int nt = 0; nt < NT; ++nt) {
+                uint2 hi, lo;
+                split_h4(scaled(accV[nt], 1.0f / SC_T), hi, lo);
+                uint16_t* dst = Vl + (SUB * nt + cl) * LD64 + SUB * wave + rl;
+                *reinterpret_cast<uint2*>(dst) = hi;
+                *reinterpret_cast<uint2*>(dst + P_PLANE) = lo;
+            }
+            KDA_LOAD_T(x, c2)
+            __syncthreads();                      // V' is in LDS
+            // Y^T = V'^T M^T + S^T Qg^T: the state and V' on the row side of the tiles, so that a lane ends up with
+            // four consecutive values of one row
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) accY[nt] = mfma_f16(frag(Vl, LD64, SUB * nt, 32, lane), as_u4(x.m[1]), accY[nt]);
+            for (int nt = 0; nt < NT; ++nt) {
+                accY[nt] = mfma_hl(frag(Vl, LD64, SUB * nt, 0, lane), frag(Vl + P_PLANE, LD64, SUB * nt, 0, lane),
+                                   as_u4(x.m[0][0]), as_u4(x.m[1][0]), zero);
+                if (nks == 2)
+                    accY[nt] = mfma_hl(frag(Vl, LD64, SUB * nt, 32, lane), frag(Vl + P_PLANE, LD64, SUB * nt, 32, lane),
+                                       as_u4(x.m[0][1]), as_u4(x.m[1][1]), accY[nt]);
             }
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
-                    accY[nt] = mfma_f16(frag(Sl, LD128, SUB * nt, 32 * ks, lane), as_u4(x.q[ks]), accY[nt]);
+                    accY[nt] = mfma_hl(frag(Sl, LD128, SUB * nt, 32 * ks, lane), frag(Sl + S_PLANE, LD128, SUB * nt, 32 * ks, lane),
+                                       as_u4(x.q[0][ks]), as_u4(x.q[1][ks]), accY[nt]);
             KDA_LOAD_QM(x, c2)
             st_c = c;
         };
         if (nch > 0) {
             ReadoutOperands xa, xb;
-            KDA_LOAD_QM(xa, 0)
+            KDA_LOAD_T(xa, 0) KDA_LOAD_QM(xa, 0)
             const int c1 = min(1, nch - 1);
-            KDA_LOAD_QM(xb, c1)
+            KDA_LOAD_T(xb, c1) KDA_LOAD_QM(xb, c1)
             int c = 0;
 #pragma unroll 1
             for (; c + 1 < nch; c += 2) {
@@ -926,6 +1040,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             if (c < nch) chunk_step(c, xa);
             store_rows();
         }
+#undef KDA_LOAD_T
 #undef KDA_LOAD_QM
     }
 }
@@ -1025,6 +1140,31 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 constexpr int kNormBlocks = 1024;
 
+
+// More than 64 KiB of LDS per workgroup is an attribute of each device's copy of a kernel: set once per device, under
+// a lock (two host threads may make their first calls together). The first call on a device therefore does more
+// than launch kernels and should come before a stream capture.
+int allow_large_lds() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex lock;
+    static bool done_on[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(lock);
+    if (done_on[dev]) return 0;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&intra_kernel<true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, INTRA_LDS) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&intra_kernel<false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, INTRA_LDS) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&inter_kernel<float>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, INTER_LDS) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&inter_kernel<bf16_t>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, INTER_LDS) != hipSuccess)
+        return (int)hipGetLastError();
+    done_on[dev] = true;
+    return 0;
+}
+
 // The passes over every sub-segment, the norm and the conv-window advance, in stream order (reference:
 // kda_prefill.cu:630-691).
 template <typename S>
@@ -1045,7 +1185,7 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
     if ((reinterpret_cast<uintptr_t>(conv_w) & 7u) || (reinterpret_cast<uintptr_t>(out) & 3u) ||
         (reinterpret_cast<uintptr_t>(g) & 3u) || (out_stride & 1) || (g_stride & 1))
         return kInvalid;
-    (void)value_blocks;   // every accepted value runs the 32-column blocks of this build
+    (void)value_blocks;   // checked as the reference checks it; this build always uses 32-column blocks
     const long long per_chunk = (long long)WS_BYTES * heads * batch;
     long long chunks = workspace_bytes / per_chunk;
     if (chunks < 1) return kInvalid;
@@ -1053,40 +1193,24 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
     if (chunks > needed) chunks = needed > 0 ? needed : 1;
     if (chunks > 65535) chunks = 65535;
     hipStream_t st = (hipStream_t)stream;
-    // The large LDS allocation is an attribute of each device's copy of a kernel: set once per device.
-    constexpr int kMaxDevices = 64;
-    static bool attr_set_on[kMaxDevices] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
-    bool& attr_set = attr_set_on[dev];
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&intra_kernel<true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, INTRA_LDS) != hipSuccess ||
-            hipFuncSetAttribute(reinterpret_cast<const void*>(&intra_kernel<false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, INTRA_LDS) != hipSuccess ||
-            hipFuncSetAttribute(reinterpret_cast<const void*>(&inter_kernel<float>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, INTER_LDS) != hipSuccess ||
-            hipFuncSetAttribute(reinterpret_cast<const void*>(&inter_kernel<bf16_t>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, INTER_LDS) != hipSuccess)
-            return (int)hipGetLastError();
-        attr_set = true;
-    }
+    const int arc = allow_large_lds();
+    if (arc != 0) return arc;
     const long long* coff = reinterpret_cast<const long long*>(conv_off);
     const long long* soff = reinterpret_cast<const long long*>(state_off);
     unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
     // 128-bit input staging needs every q | k | v and gate row segment on a 16-byte boundary (the model's strides
     // are); other layouts take the 16-bit path. Conv-window offsets are device data: whole windows keep alignment.
     const int vec = aligned16(p) && aligned16(a) && aligned16(conv) && (p_stride % 8 == 0) && (a_stride % 8 == 0);
-    const int step = (int)chunks * CH;
-    for (int sub0 = 0; sub0 == 0 || sub0 < max_rows; sub0 += step) {
+    const long long step = chunks * CH;
+    for (long long sub0 = 0; sub0 == 0 || sub0 < max_rows; sub0 += step) {
         if (max_rows > 0) {
             const dim3 grid((unsigned)((chunks + INTRA_CPW - 1) / INTRA_CPW), heads, batch);
             if (vec)
-                intra_kernel<true><<<grid, THREADS, INTRA_LDS, st>>>(heads, cu_rows, rows1, sub0, (int)chunks, bfp(p),
+                intra_kernel<true><<<grid, THREADS, INTRA_LDS, st>>>(heads, cu_rows, rows1, (int)sub0, (int)chunks, bfp(p),
                                                                      p_stride, b_off, bfp(a), a_stride, bfp(conv), coff,
                                                                      bfp(conv_w), a_log, dt_bias, lower, ws);
             else
-                intra_kernel<false><<<grid, THREADS, INTRA_LDS, st>>>(heads, cu_rows, rows1, sub0, (int)chunks, bfp(p),
+                intra_kernel<false><<<grid, THREADS, INTRA_LDS, st>>>(heads, cu_rows, rows1, (int)sub0, (int)chunks, bfp(p),
                                                                       p_stride, b_off, bfp(a), a_stride, bfp(conv), coff,
                                                                       bfp(conv_w), a_log, dt_bias, lower, ws);
             const int rc = (int)hipGetLastError();
@@ -1094,7 +1218,7 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
         }
         const S* s_in = sub0 == 0 ? state_in : state_out;
         inter_kernel<S><<<dim3(heads * VBLOCKS, batch), INTER_THREADS, INTER_LDS, st>>>(
-            heads, cu_rows, rows1, sub0, (int)chunks, s_in, state_out, soff, bfp(out), out_stride, ws);
+            heads, cu_rows, rows1, (int)sub0, (int)chunks, s_in, state_out, soff, bfp(out), out_stride, ws);
         const int rc = (int)hipGetLastError();
         if (rc != 0) return rc;
         if (max_rows == 0) break;

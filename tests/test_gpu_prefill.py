@@ -248,10 +248,10 @@ def test_bad_arguments_are_rejected():
     sr = hs.StagedRows(rows)
     conv_d, s_d = hs.to_bf16(conv), hs.to_f32(s0)
     ws_bytes = ffi.glm53f_kda_prefill_workspace_bytes(heads, 1, 64)
-    assert ws_bytes == 74240 * heads
+    assert ws_bytes == 147968 * heads
     assert ffi.glm53f_kda_prefill_workspace_bytes(0, 1, 64) == 0
     assert ffi.glm53f_kda_prefill_workspace_bytes(heads, 1, 0) == 0
-    assert ffi.glm53f_kda_prefill_workspace_bytes(heads, 2, 65) == 2 * 2 * 74240 * heads
+    assert ffi.glm53f_kda_prefill_workspace_bytes(heads, 2, 65) == 2 * 2 * 147968 * heads
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=hs.DEV)
 
     def call(vb=0, state_out=True, lower=None, wsb=ws_bytes, heads_=heads):
