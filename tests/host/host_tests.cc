@@ -137,7 +137,9 @@ static void cpu_tests() {
     PrefillWorkspace ws;
     ws.heads = h; ws.batch = 2; ws.rows_per_pass = 128;
     ws.buf = fake(0xb00000, PrefillWorkspace::bytes_for(h, 2, 128));
-    EXPECT(ws.buf.bytes == 2 * 2 * 74240 * h);
+    // two chunks of two requests: linear in chunks, requests and heads
+    EXPECT(ws.buf.bytes == 2 * 2 * h * (size_t)glm53f_kda_prefill_workspace_bytes(1, 1, PREFILL_CHUNK));
+    EXPECT(glm53f_kda_prefill_workspace_bytes(1, 1, PREFILL_CHUNK) > 0);
     Prefill pf;
     pf.weights = &w; pf.rows = rows; pf.p = RowView(p, 0, ps); pf.b_off = (int64_t)c; pf.a = RowView::dense(a, h * DK);
     pf.g = RowView::dense(g, h * DV); pf.conv = conv; pf.state = state; pf.state_out = StateOut::in_place();
@@ -316,7 +318,9 @@ static void gpu_tests() {
     // Prefill through the wrapper against the literal recurrence
     PrefillWorkspace ws;
     EXPECT_OK(PrefillWorkspace::within(h, 1, 1 << 20, &ws));
-    EXPECT(ws.rows_per_pass == 192);
+    // the largest whole number of chunks whose workspace fits the budget, by the library's own figure per chunk
+    EXPECT(ws.rows_per_pass == ((size_t)(1 << 20) / (size_t)glm53f_kda_prefill_workspace_bytes((int32_t)h, 1, PREFILL_CHUNK)) * PREFILL_CHUNK);
+    EXPECT(ws.rows_per_pass >= PREFILL_CHUNK);
     EXPECT_OK(d_state.upload(s0));
     EXPECT_OK(d_conv.upload(enc(conv)));
     Prefill pf;
