@@ -356,7 +356,21 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                     acc = dot2_bf16(x1, w[1], acc);
                     acc = dot2_bf16(x2, w[2], acc);
                     acc = dot2_bf16(x3, w[3], acc);
-                    s2[k] = acc * fast_sigmoid(acc);
+                    // SiLU as the quotient acc / (1 + e^-acc), the reference's form: the hardware reciprocal's
+                    // product is corrected by one residual step (two fused operations), which makes it the
+                    // correctly rounded quotient in all but a few cases per million. The plain product
+                    // acc * rcp(1 + e^-acc) put one conv output in 150,000 on the other side of its bf16 rounding
+                    // than the host's quotient (the chain kernel, with a true division: one in 700,000; so does
+                    // this), and every such value in a row that decay has not yet forgotten moves the head's state
+                    // by 2^-9 of a value: 5e-4 of the state where decay is slow.
+                    {
+                        // (Below -88.7 the exponential is infinite and the quotient -0, as on the host: the
+                        // residual takes the largest finite number in its place, or it would be 0 x inf.)
+                        const float dd = 1.0f + fast_exp(-acc);
+                        const float y = fast_rcp(dd);
+                        const float q0 = acc * y;
+                        s2[k] = __builtin_fmaf(__builtin_fmaf(-q0, fminf(dd, 3.4028234663852886e38f), acc), y, q0);
+                    }
                 }
                 const uint32_t pair = f2bf2(s2[0], s2[1]);        // the one bf16 rounding
                 if (seg == 0) { qr[4 * p + d] = pair; ssq = dot2_bf16(pair, pair, ssq); }

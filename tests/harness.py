@@ -259,6 +259,15 @@ def ulps(a, b):
     return int(d.max()) if d.size else 0, int((d > 0).sum())
 
 
+def bf16_state_close(got, ref, share=1e-3):
+    """A bf16-stored state against the CPU model with the same rounding points: the device's exp, division and square
+    root differ from the host's in the last place, which flips an isolated bf16 rounding now and then. So: within one
+    bf16 step of the largest entry everywhere, and at most `share` of the entries differ at all."""
+    got, ref = np.asarray(got, np.float32), np.asarray(ref, np.float32)
+    differ = int((bits(got) != bits(ref)).sum())
+    return rel_err(got, ref) <= 2.0 ** -8 and differ <= max(2, share * got.size)
+
+
 def bf16_steps(a, b):
     """How many representable bf16 values apart two arrays of bf16-valued floats are."""
     def key(x):
@@ -308,3 +317,42 @@ def prefill_gpu(p: o.LayerParams, conv: np.ndarray, state: np.ndarray, rows: o.R
     check(code, "prefill")
     sync()
     return sr.out_np(), back(s_out), back(conv_d)
+
+
+# --------------------------------------------------------------------------------------- head subsets
+# Heads are independent (state, conv channels, norms and gates are per head), so a run over H heads restricted to a
+# few of them equals a run of the oracle over just those: what makes the full-size configurations checkable on the
+# host in seconds.
+
+def subset_params(p: o.LayerParams, heads: list[int]) -> o.LayerParams:
+    h = p.heads
+    cw = np.asarray(p.conv_w, np.float32).reshape(3, h, DK, 4)[:, heads].reshape(-1)
+    return o.LayerParams(len(heads), cw, np.asarray(p.a_log, np.float32)[heads],
+                         np.asarray(p.dt_bias, np.float32).reshape(h, DK)[heads].reshape(-1), p.norm_w, p.eps, p.lower)
+
+
+def subset_rows(h: int, heads: list[int], P: torch.Tensor, A: torch.Tensor, G: torch.Tensor, r0: int, r1: int) -> o.Rows:
+    """Rows r0..r1 of device buffers in the engine's layout (p rows of C + H columns, dense a and g), the chosen
+    heads only, as oracle rows on the host."""
+    c, n = channels(h), r1 - r0
+    idx = torch.tensor(heads, device=P.device)
+    qkv = P[r0:r1, :c].reshape(n, 3, h, DK).index_select(2, idx).float().cpu().numpy().reshape(-1)
+    b = P[r0:r1, c:c + h].index_select(1, idx).float().cpu().numpy().reshape(-1)
+    a = A[r0:r1].reshape(n, h, DK).index_select(1, idx).float().cpu().numpy().reshape(-1)
+    g = G[r0:r1].reshape(n, h, DV).index_select(1, idx).float().cpu().numpy().reshape(-1)
+    return o.Rows(len(heads), n, qkv, a, b, g)
+
+
+def subset_conv(h: int, heads: list[int], window: torch.Tensor) -> np.ndarray:
+    idx = torch.tensor(heads, device=window.device)
+    return window.reshape(WINDOW, 3, h, DK).index_select(2, idx).float().cpu().numpy().reshape(-1)
+
+
+def subset_state(h: int, heads: list[int], state: torch.Tensor) -> np.ndarray:
+    idx = torch.tensor(heads, device=state.device)
+    return state.reshape(h, DV * DK).index_select(0, idx).float().cpu().numpy().reshape(-1)
+
+
+def subset_out(h: int, heads: list[int], out: torch.Tensor) -> np.ndarray:
+    idx = torch.tensor(heads, device=out.device)
+    return out.reshape(out.shape[0], h, DV).index_select(1, idx).float().cpu().numpy().reshape(-1)

@@ -79,10 +79,10 @@ def test_gpu_chain_meets_the_vectors(vec):
     assert hs.max_rel(g.saves.g, vec["chain.save_g"]) <= 4e-6
     assert hs.ulps(g.saves.v, vec["chain.save_v"])[0] <= 1 and hs.ulps(g.saves.beta, vec["chain.save_beta"])[0] <= 1
     assert hs.max_abs(g.saves.k, vec["chain.save_k"]) <= 1.0 / 256.0
-    assert hs.rel_err(g.state, vec["chain.state_out"]) <= 1e-3
+    assert hs.rel_err(g.state, vec["chain.state_out"]) <= 1e-5
     assert hs.rel_err(g.out, vec["chain.out"]) <= 1.0 / 256.0
     # The north-star bars against the FP32 recurrent reference.
-    assert hs.rel_err(g.state, vec["chain.literal_state"]) <= 1e-3
+    assert hs.rel_err(g.state, vec["chain.literal_state"]) <= 1e-5
     assert hs.max_abs(g.out, vec["chain.literal_out"]) <= 2e-2
     # Replay of the fixture's saves and the conv shift involve no transcendental function: bitwise.
     sv = hs.Saves(heads, rows.rows)
@@ -112,7 +112,7 @@ def test_gpu_bf16_state_chain_meets_the_vectors(vec):
     # state may differ by a bf16 rounding flip where exp differs in the last place (tests/gpu_bf16_state.rs:385-419).
     got = pool.device_state(0, s_out)
     assert same_bits(o.replay(s0, sv.download(rows.rows), rows.rows, bf16_state=True), got)
-    assert hs.rel_err(got, vec["chain16.state_out"]) <= 1e-2
+    assert hs.bf16_state_close(got, vec["chain16.state_out"])
     assert hs.rel_err(out, vec["chain16.out"]) <= 1.0 / 256.0
 
 
@@ -122,9 +122,9 @@ def test_gpu_prefill_meets_the_vectors(vec):
 
     p, conv, s0, rows = case(vec, "prefill")
     out, state, conv_after = hs.prefill_gpu(p, conv, s0, rows)
-    assert hs.rel_err(state, vec["prefill.state_out"]) <= 1e-3
-    # 2e-2, or two representable bf16 values where those are further apart than that (outputs beyond 2): the
-    # read-out and the gated norm each round to bf16, so a last-place difference can move an output two steps.
-    far = np.abs(out - vec["prefill.out"]) > 2e-2
-    assert not far.any() or hs.bf16_steps(out, vec["prefill.out"])[far].max() <= 2
+    assert hs.rel_err(state, vec["prefill.state_out"]) <= 1e-5
+    # the synthetic layer's outputs reach 7, where one bf16 step is 3e-2: normwise two steps of the largest output,
+    # and only a handful of outputs may differ at all
+    assert hs.rel_err(out, vec["prefill.out"]) <= 2.0 ** -7
+    assert hs.ulps(out, vec["prefill.out"])[1] <= max(4, 0.003 * out.size)
     assert same_bits(conv_after, vec["prefill.conv_after"])

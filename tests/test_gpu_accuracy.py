@@ -5,7 +5,7 @@ tests/gpu_bf16_state.rs:704-804 (drift over 8K and 64K rows): final states again
 replay inputs (so every path sees the same k, v, decay and beta), with gates across the whole range and with every
 channel decaying slowly (multipliers of at least 0.9993, where old rounding is forgotten mostly through the delta
 rule itself). The reference's prefill is f32 throughout and is held to 1e-6 there; this one feeds the matrix cores
-fp16 operands and is held to the north-star bound of 1e-3, with the measured figures printed.
+fp16 hi/lo pairs (22 bits) and is held to 2.5e-4, a quarter of the north-star bound, with the measured figures printed.
 """
 import numpy as np
 import pytest
@@ -19,7 +19,8 @@ import harness as hs
 pytestmark = pytest.mark.gpu
 
 H, SEG = 8, 8192
-STATE_TOL = 1e-3
+STATE_TOL = 2.5e-4        # measured: 2.7e-6 with gates across the range, 9.7e-5 with slow decay over 8192 rows (the
+                         # operands carry 22 bits, not f32's 24, and slow decay forgets no rounding); north-star bar 1e-3
 
 
 def layer(slow):

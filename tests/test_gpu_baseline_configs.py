@@ -2,8 +2,9 @@
 
 Config 1 (decode, 16 of 48 slots) lives in test_gpu_chain.py. Here: config 2 (T = 8192 as four 2048-row calls)
 against the FP32 recurrent oracle with the north-star tolerances; config 3 (varlen packed prefill) at a size the
-oracle finishes in seconds and, at its full 131072 / 20480 / 4096 / 777 rows, through properties that do not
-depend on the size (packed == per request bit for bit, conv windows exact); config 4 (verify 48 slots x 16
+oracle finishes in seconds for all heads and at its full 131072 / 20480 / 4096 / 777 rows: values of four heads
+against the oracle from restored snapshots, and properties that do not depend on the size (packed == per request
+bit for bit, conv windows exact); config 4 (verify 48 slots x 16
 drafts with checkpoints) against serial decode steps, bit for bit.
 """
 import numpy as np
@@ -18,23 +19,30 @@ import harness as hs
 pytestmark = pytest.mark.gpu
 
 
-def check_outputs(got, ref, label):
-    """The north-star bar on bf16 outputs is max-abs <= 2e-2, which is what two bf16 steps come to for outputs
-    below 2 (2 * 2^-7 = 1.56e-2). The contract rounds twice (the read-out to bf16, then the gated norm's result to
-    bf16), so a difference far below any tolerance that flips the read-out's rounding moves the output by one step
-    and the output's own rounding can add another: two steps is the floor for every kernel that is not bit-exact,
-    the reference's CUDA chain against its CPU model included. Two steps exceed 2e-2 from 2 upwards (and for a pair
-    that straddles 2), and outputs reach 6 to 7 over 67 million draws, so every output must satisfy
-    |diff| <= 2e-2 or be at most two representable values away; the print says how many needed the second clause."""
+def check_outputs(got, ref, label, flip_fraction=0.003):
+    """The north-star bar on bf16 outputs: max-abs <= 2e-2 against the FP32 recurrent oracle. The contract rounds
+    twice (the read-out to bf16, then the gated norm's result to bf16), so an output whose read-out lands on the
+    other side of a rounding boundary moves one or two representable values, and two values are 3.1e-2 apart from
+    |out| = 2 upwards: for any kernel that is not bit-exact the bar holds only while such flips are rare. With every
+    operand at f32-class precision 0.055 % of the outputs differ at all (the reference's kernel: 0.013 %, its bar
+    0.1 %, gpu_prefill.rs:270-276; this build's f32 chain kernel: 0.024 %), which leaves a two-step event at
+    |out| >= 2 about once in 10^8 outputs: none among the 67 million of config 2, one among the 80 million checked of
+    config 3. So: every output within 2e-2, except that one output per array (and one more per 30 million) may be
+    two representable values away where those are further apart than that; and the share that differs at all is
+    bounded."""
     got, ref = np.asarray(got, np.float32), np.asarray(ref, np.float32)
     d = np.abs(got.astype(np.float64) - ref.astype(np.float64))
     steps = hs.bf16_steps(got, ref)
     hist = np.bincount(np.minimum(steps, 4).ravel(), minlength=5)
+    differ = int((steps > 0).sum())
     over = d > 2e-2
-    print(f"{label}: outputs 0/1/2/3/4+ bf16 steps apart: {hist.tolist()}; {int(over.sum())} differ by more than 2e-2 "
-          f"(all at |out| >= {float(np.abs(ref[over]).min()) if over.any() else 0:.3f}), worst of those "
-          f"{int(steps[over].max()) if over.any() else 0} steps")
-    assert int(steps[over].max() if over.any() else 0) <= 2, label
+    print(f"{label}: out max-abs {float(d.max()) if d.size else 0.0:.3e}; outputs 0/1/2/3/4+ bf16 steps apart: "
+          f"{hist.tolist()}; {differ} of {got.size} differ ({100.0 * differ / max(got.size, 1):.4f} %); "
+          f"{int(over.sum())} by more than 2e-2")
+    assert int(over.sum()) <= 1 + got.size // 30_000_000, label
+    if over.any():
+        assert int(steps[over].max()) <= 2 and float(np.minimum(np.abs(got[over]), np.abs(ref[over])).min()) >= 1.9, label
+    assert differ <= max(4, flip_fraction * got.size), label
 
 
 def baseline_layer(heads, seed):
@@ -72,9 +80,9 @@ def test_baseline_config2_prefill_8192_in_four_lanes():
     lit = o.literal_chain(p, conv0, s0, rows, threads=16)
     es, ea = hs.rel_err(st, lit.state), hs.max_abs(out, lit.out)
     _, nd = hs.ulps(out, lit.out)
-    print(f"config 2: state {es:.2e} rel (bar 1e-3); out max-abs {ea:.2e}, {nd}/{out.size} differ; "
-          f"max |out| {np.max(np.abs(lit.out)):.2f}")
-    assert es <= 1e-3
+    print(f"config 2: state {es:.2e} rel (north-star bar 1e-3, the reference's own 1e-5); out max-abs {ea:.2e}, "
+          f"{nd}/{out.size} differ; max |out| {np.max(np.abs(lit.out)):.2f}")
+    assert es <= 1e-5
     check_outputs(out, lit.out, "config 2")
     assert np.array_equal(conv, o.conv_shift(conv0, rows, total))
 
@@ -111,7 +119,9 @@ def test_baseline_config3_varlen_packed_against_the_oracle_reduced():
               f"differ (max {u} ulp), raw {raw:.2e} rel; out max-abs {ea:.2e}")
         assert raw <= 2.0 ** -8                      # bf16 storage (2^-9) on top of the 1e-3 bar
         assert hs.rel_err(got, o.bf16_round(lit.state)) <= 2.0 ** -8
-        check_outputs(out[r0 * n:(r0 + rq.rows) * n], lit.out, f"config 3 (reduced), request {i}")
+        # the state of this entry point is bf16 between chunks, the oracle's is f32 throughout: the read-outs differ
+        # by the state's rounding (2^-9), which moves a percent of them across a bf16 boundary
+        check_outputs(out[r0 * n:(r0 + rq.rows) * n], lit.out, f"config 3 (reduced), request {i}", flip_fraction=0.03)
         pool1 = hs.Pool(heads, 5, True, 3020)
         pool1.state, pool1.conv = hs.to_bf16(pool.state_host), hs.to_bf16(pool.conv_host)
         o1, _, _ = hs.prefill_batch_gpu(p, pool1, [slot], [rq], write="inplace", rows_per_pass=512)
@@ -175,6 +185,149 @@ def test_baseline_config3_varlen_packed_full_size_properties():
         # the window is exactly the request's last three q|k|v rows
         assert torch.equal(cv[s * cw:(s + 1) * cw].view(WINDOW, c), P[cu[i + 1] - 3:cu[i + 1], :c]), f"request {i}: window rows"
         del o1, s1, c1
+
+
+def test_baseline_config3_full_size_values_from_a_restored_snapshot():
+    """Config 3 as the benchmark definition states it: 131072 + 20480 + 4096 + 777 rows packed, 64 heads, f32 carried
+    state, initial states from a prior-prefix snapshot, bf16 final states written back to the slot pool. The
+    snapshot is real: a prefix of every prompt is prefilled into the pool's slots, saved as a mark, the slots are
+    overwritten, and the marks are loaded back (the row scatter / gather of the snapshot path) before the prompts
+    continue. Values: heads 0, 21, 42 and 63 of every request against the FP32 recurrent oracle run on those heads
+    alone (heads are independent), states and every output row, under the north-star bars."""
+    from glm53f_forward.kv import KvPool
+    from glm53f_forward.kvplan import KvLayout
+
+    heads, lens, prefix, slots = 64, [131072, 20480, 4096, 777], [300, 200, 64, 37], [2, 0, 3, 1]
+    sub = [0, 21, 42, 63]
+    c, n, cw = channels(heads), state_len(heads), WINDOW * channels(heads)
+    total, ps = sum(lens), c + heads
+    gen = torch.Generator(device=hs.DEV).manual_seed(33)
+    p = baseline_layer(heads, 3300)
+    w = hs.Weights(p)
+
+    def draw(rows):
+        P = torch.empty(rows, ps, device=hs.DEV, dtype=torch.bfloat16)
+        A = torch.empty(rows, heads * DK, device=hs.DEV, dtype=torch.bfloat16)
+        G = torch.empty(rows, heads * DV, device=hs.DEV, dtype=torch.bfloat16)
+        for r0 in range(0, rows, 16384):       # in slices: the f32 temporaries stay small
+            r1 = min(rows, r0 + 16384)
+            P[r0:r1] = torch.randn(r1 - r0, ps, device=hs.DEV, generator=gen).to(torch.bfloat16)
+            sp = torch.clamp(torch.nn.functional.softplus(torch.randn(r1 - r0, heads * DK, device=hs.DEV, generator=gen)), max=4.999)
+            A[r0:r1] = (torch.log(sp / 5.0) - torch.log1p(-sp / 5.0)).to(torch.bfloat16)
+            G[r0:r1] = torch.randn(r1 - r0, heads * DV, device=hs.DEV, generator=gen).to(torch.bfloat16)
+        return P, A, G
+
+    # the pool: one KDA layer, bf16 states, five slots
+    layout = KvLayout(kda_layers=1, dsa_layers=1, kda_state_bf16=True)
+    pool = KvPool(layout, slots=5, pages=4 * layout.mark_pages() + 3)
+    kvs = [pool.slot() for _ in range(5)]
+    state16, conv16 = pool.state.view(torch.bfloat16), pool.conv.view(torch.bfloat16)
+    conv16[:] = torch.randn(5 * cw, device=hs.DEV, generator=gen).to(torch.bfloat16)
+    conv_start = conv16.clone()
+    soff = [kvs[s].state_at() // 2 for s in slots]       # element offsets of the slots' regions
+    coff = [kvs[s].conv_at() // 2 for s in slots]
+    assert soff == [s * n for s in slots] and coff == [s * cw for s in slots]
+
+    # 1. the prior prefixes, from empty slots, with the bf16 state of the pool
+    Pp, Ap, Gp = draw(sum(prefix))
+    outp = torch.zeros(sum(prefix), heads * DV, device=hs.DEV, dtype=torch.bfloat16)
+    meta_p = hs.BatchMeta(prefix, coff, soff)
+    ws_bytes = ffi.glm53f_kda_prefill_workspace_bytes(heads, 4, 1024)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=hs.DEV)
+    hs.check(ffi.glm53f_kda_prefill_batch_bf16state(
+        heads, 4, hs.ptr(meta_p.cu_rows), max(prefix), hs.ptr(Pp), ps, c, hs.ptr(Ap), heads * DK, hs.ptr(Gp), heads * DV,
+        hs.ptr(conv16), hs.ptr(meta_p.conv_off), hs.ptr(w.conv_w), hs.ptr(state16), hs.ptr(state16),
+        hs.ptr(meta_p.state_off), *w.args(), hs.ptr(outp), heads * DV, 0, hs.ptr(ws), ws_bytes, None), "prefix prefill")
+    hs.sync()
+    cup = np.concatenate([[0], np.cumsum(prefix)])
+    p4 = hs.subset_params(p, sub)
+    for i, s in enumerate(slots):
+        pre = hs.subset_rows(heads, sub, Pp, Ap, Gp, int(cup[i]), int(cup[i + 1]))
+        lit = o.literal_chain(p4, hs.subset_conv(heads, sub, conv_start[s * cw:(s + 1) * cw]),
+                              np.zeros(state_len(4), np.float32), pre, threads=4)
+        got = hs.subset_state(heads, sub, state16[s * n:(s + 1) * n])
+        # a bf16 state rounded after every chunk against the unrounded oracle: the storage format's bound
+        assert hs.rel_err(got, lit.state) <= 2.0 ** -7, f"prefix of request {i}"
+
+    # 2. mark, overwrite, rewind: the prompts continue from restored snapshots
+    saved_state, saved_conv = state16.clone(), conv16.clone()
+    marks = []
+    for i, s in enumerate(slots):
+        kvs[s].tokens = prefix[i]
+        marks.append(kvs[s].mark())
+    state16[:] = torch.randn(5 * n, device=hs.DEV, generator=gen).to(torch.bfloat16)
+    conv16[:] = torch.randn(5 * cw, device=hs.DEV, generator=gen).to(torch.bfloat16)
+    for i, s in enumerate(slots):
+        kvs[s].tokens = prefix[i] + 5
+        kvs[s].rewind(prefix[i], marks[i])
+    hs.sync()
+    for s in slots:
+        assert torch.equal(state16[s * n:(s + 1) * n], saved_state[s * n:(s + 1) * n]), f"slot {s}: restored state"
+        assert torch.equal(conv16[s * cw:(s + 1) * cw], saved_conv[s * cw:(s + 1) * cw]), f"slot {s}: restored window"
+    del Pp, Ap, Gp, outp, saved_state, saved_conv
+
+    # 3. the packed prompts with an f32 carried state, bf16 states back into the pool
+    P, A, G = draw(total)
+    out = torch.zeros(total, heads * DV, device=hs.DEV, dtype=torch.bfloat16)
+    conv_before = conv16.clone()
+    state32 = state16.float()
+    state_before = state32.clone()
+    meta = hs.BatchMeta(lens, coff, soff)
+    assert list(meta.cu_host) == [0, 131072, 151552, 155648, 156425]
+    ws_bytes = ffi.glm53f_kda_prefill_workspace_bytes(heads, 4, 2048)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=hs.DEV)
+    hs.check(ffi.glm53f_kda_prefill_batch(
+        heads, 4, hs.ptr(meta.cu_rows), max(lens), hs.ptr(P), ps, c, hs.ptr(A), heads * DK, hs.ptr(G), heads * DV,
+        hs.ptr(conv16), hs.ptr(meta.conv_off), hs.ptr(w.conv_w), hs.ptr(state32), hs.ptr(state32),
+        hs.ptr(meta.state_off), *w.args(), hs.ptr(out), heads * DV, 0, hs.ptr(ws), ws_bytes, None), "prefill_batch")
+    hs.sync()
+    state16.copy_(state32.to(torch.bfloat16))              # the write-back to the slot pool
+    cu = meta.cu_host
+    for i, s in enumerate(slots):
+        r0, r1 = int(cu[i]), int(cu[i + 1])
+        rq = hs.subset_rows(heads, sub, P, A, G, r0, r1)
+        lit = o.literal_chain(p4, hs.subset_conv(heads, sub, conv_before[s * cw:(s + 1) * cw]),
+                              hs.subset_state(heads, sub, state_before[s * n:(s + 1) * n]), rq, threads=4)
+        got32 = hs.subset_state(heads, sub, state32[s * n:(s + 1) * n])
+        got16 = hs.subset_state(heads, sub, state16[s * n:(s + 1) * n])
+        es = hs.rel_err(got32, lit.state)
+        u, nd = hs.ulps(got16, o.bf16_round(lit.state))
+        print(f"config 3, request {i} ({lens[i]} rows, heads {sub}): f32 state {es:.2e} rel (bar 1e-3); pool state vs "
+              f"bf16(f32 oracle): {nd} of {got16.size} differ, max {u} ulp; raw {hs.rel_err(got16, lit.state):.2e} rel")
+        # Per head. The conv's one bf16 rounding falls the other way on the device than on the host for about one
+        # channel value in 10^5 (SiLU through the hardware's exp and reciprocal; the reference notes the same of its
+        # kernels, tests/gpu.rs:326-331). Such a value in one of a prompt's last rows, before decay has forgotten it,
+        # moves that head's state by up to 2^-9 of a value row times beta: measured 2.2e-4 on one head of the long
+        # prompt, 1e-6 on every other. So: the north-star bar on every head, f32-class on the typical one.
+        per = [hs.rel_err(got32.reshape(len(sub), -1)[j], lit.state.reshape(len(sub), -1)[j]) for j in range(len(sub))]
+        print(f"    per head: {[f'{e:.1e}' for e in per]}")
+        assert es <= 1e-3 and float(np.median(per)) <= 1e-5, i
+        assert nd <= 2e-3 * got16.size, i                      # roundings that fall the other way
+        assert hs.rel_err(got16, lit.state) <= 2.0 ** -8, i    # one rounding to bf16
+        check_outputs(hs.subset_out(heads, sub, out[r0:r1]), lit.out, f"config 3, request {i}")
+        # the window a request leaves is its last three q | k | v rows
+        assert torch.equal(conv16[s * cw:(s + 1) * cw].view(WINDOW, c), P[r1 - 3:r1, :c]), i
+    # the slot no request lives in is untouched
+    free = (set(range(5)) - set(slots)).pop()
+    assert torch.equal(state32[free * n:(free + 1) * n], state_before[free * n:(free + 1) * n])
+
+
+def test_baseline_config0_shape_through_the_prefill():
+    """Config 0's shape (one sequence, T = 256, 64 heads, zero initial state, g = -softplus(N(0, 1)) through the
+    lower-bound gate) through the prefill kernels against the literal recurrence; config 0 itself (core-level
+    inputs, chunked against recurrent on the CPU) is in test_oracle.py."""
+    heads, t = 64, 256
+    p = baseline_layer(heads, 100)
+    rows = baseline_rows(heads, t, 101)
+    conv0 = o.bf16_round(np.random.default_rng(102).standard_normal(WINDOW * channels(heads), dtype=np.float32))
+    s0 = np.zeros(state_len(heads), np.float32)
+    out, st, conv = hs.prefill_gpu(p, conv0, s0, rows, rows_per_pass=256)
+    lit = o.literal_chain(p, conv0, s0, rows, threads=16)
+    es = hs.rel_err(st, lit.state)
+    print(f"config 0 shape: state {es:.2e} rel")
+    assert es <= 1e-5
+    check_outputs(out, lit.out, "config 0 shape")
+    assert np.array_equal(conv, o.conv_shift(conv0, rows, t))
 
 
 def test_baseline_config4_verify_checkpoints_and_rollback():

@@ -1,10 +1,10 @@
 """The chunked prefill on the GPU against the CPU oracle, through the C ABI.
 
 Follows the reference's prefill tests (crates/glm53f-kda/tests/gpu_prefill.rs:245-651,
-tests/gpu_bf16_state.rs:592-656) with this build's tolerances: the matrix-core form feeds the state with
-fp16 / split-bf16 operands, so it agrees with the FP32 recurrent reference to 1e-3 on the state (normwise)
-and to a bf16 rounding on the outputs, not to f32 rounding as the reference's CUDA-core kernel does. Indexing
-(batching, slots, ragged tails, workspace size, conv windows) is bit-exact.
+tests/gpu_bf16_state.rs:592-656) with the reference's own bars: every matrix-core operand is an fp16 hi/lo
+pair (22 significant bits), so the f32 state agrees with the FP32 recurrent reference to 1e-5 normwise
+(gpu_prefill.rs:245-247) and only a fraction of a percent of the bf16 outputs land on the other side of a rounding
+boundary. Indexing (batching, slots, ragged tails, workspace size, conv windows) is bit-exact.
 """
 import numpy as np
 import pytest
@@ -17,10 +17,17 @@ import harness as hs
 
 pytestmark = pytest.mark.gpu
 
-STATE_TOL = 1e-3          # max |diff| / max |ref| against the FP32 recurrent reference
+STATE_TOL = 1e-5          # f32 state, max |diff| / max |ref| against the FP32 recurrent reference (measured <= 3e-6)
+BF16_STATE_TOL = 2.0 ** -7  # a bf16-stored state against the unrounded f32 reference: the storage format's 2^-9 per
+                          # rounding, a few roundings deep (the reference's own bound is 1e-2, gpu_bf16_state.rs:414)
 OUT_REL = 2.0 ** -7       # bf16 outputs, normwise: the reference's own bound (gpu_prefill.rs:245-247)
 OUT_ABS = 2e-2            # bf16 outputs, max-abs, on the benchmark definition's distributions (outputs of order one)
-FLIP_FRACTION = 0.25      # at most this share of outputs may differ at all
+FLIP_FRACTION = 0.003     # at most this share of outputs may differ at all (measured <= 0.1 %; reference: 0.1 %)
+
+
+def flips_ok(differ, size):
+    """A handful of outputs is allowed whatever the size: 0.3 % of a one-row request is less than two values."""
+    return differ <= max(4, FLIP_FRACTION * size)
 
 
 def out_ok(got, ref):
@@ -52,7 +59,7 @@ def check_against_oracle(p, conv, s0, rows, out, st, cv, label):
     print(f"{label}: state {es:.2e} rel; out max-abs {ea:.2e}, {nd}/{out.size} differ")
     assert es <= STATE_TOL, label
     assert out_ok(out, lit.out), label
-    assert nd <= FLIP_FRACTION * out.size, label
+    assert flips_ok(nd, out.size), label
     assert np.array_equal(cv, o.conv_shift(conv, rows, rows.rows)), label
     assert np.all(np.isfinite(st))
 
@@ -168,14 +175,11 @@ def test_random_ragged_batches_against_the_oracle(seed):
             continue
         lit = o.literal_chain(p, pool.conv_of(slot), pool.state_of(slot), rq, threads=8)
         assert np.all(np.isfinite(got)), (label, i)
-        assert hs.rel_err(got, lit.state) <= (2.0 ** -7 if bf16_state else STATE_TOL), (label, i)
-        # Requests of a few rows have no large output to hide behind: where the bf16 read-out `y` lands on the
-        # other side of a rounding boundary (one step, up to 2^-7 of the value), the gated norm's own rounding can
-        # make it two steps of the output, so the normwise bound here is 2^-6 and the share of outputs that differ
-        # at all stays bounded as in the fixed cases.
+        assert hs.rel_err(got, lit.state) <= (BF16_STATE_TOL if bf16_state else STATE_TOL), (label, i)
+        # normwise 2^-7: two bf16 steps of the largest output (the read-out and the gated norm each round to bf16)
         got_rows, ref_rows = out[r0 * n:(r0 + rq.rows) * n], lit.out
-        assert hs.rel_err(got_rows, ref_rows) <= 2.0 ** -6, (label, i)
-        assert hs.ulps(got_rows, ref_rows)[1] <= FLIP_FRACTION * got_rows.size, (label, i)
+        assert hs.rel_err(got_rows, ref_rows) <= OUT_REL, (label, i)
+        assert bf16_state or flips_ok(hs.ulps(got_rows, ref_rows)[1], got_rows.size), (label, i)
     for slot in set(range(slots_n)) - set(slots):
         at = pool.conv_off(slot)
         assert np.array_equal(hs.back(pool.conv[at:at + cw]), pool.conv_of(slot)), (label, slot)
@@ -272,3 +276,48 @@ def test_bad_arguments_are_rejected():
     for vb in (1, 2, 4):
         assert call(vb=vb) == 0
     hs.sync()
+
+
+def test_magnitudes_the_fp16_pairs_carry():
+    """The state, V - Kd S and V' pass through the matrix cores as fp16 pairs with scale 4, so their magnitudes must
+    stay below 65,504 / 4 = 16,376 and they carry an absolute error floor of 2^-25 / 4 = 7.5e-9 (the f32 kernels of
+    the reference have neither limit). |Kd S| is at most the 2-norm of a value row of the state (the keys are unit
+    vectors), so states up to 16,376 / sqrt(128) = 1,400 in magnitude are safe whatever the keys. Inside the
+    domain: f32-class results for states of several hundred and values of a hundred, and for states and values of
+    1e-5. Beyond it the state becomes non-finite - visibly, not a finite wrong value - where the recurrence stays
+    finite."""
+    heads, t = 4, 150
+    p, conv, _, rows = case(heads, t, 7700)
+    c = channels(heads)
+    # large: |S| up to 800, conv inputs of the values up to a hundred (SiLU's exponential overflows below -88.7)
+    big = o.Rows(heads, t, rows.qkv.copy(), rows.a, rows.b, rows.gate)
+    qkv = big.qkv.reshape(t, 3, heads * DK)
+    qkv[:, 2] = o.bf16_round(qkv[:, 2] * 32.0)
+    conv_big = conv.copy().reshape(WINDOW, 3, heads * DK)
+    conv_big[:, 2] = o.bf16_round(conv_big[:, 2] * 32.0)
+    s_big = o.synth_state(heads, 7701, 800.0)
+    out, st, _ = hs.prefill_gpu(p, conv_big.reshape(-1), s_big, big)
+    lit = o.literal_chain(p, conv_big.reshape(-1), s_big, big, threads=8)
+    print(f"large: max |S| {np.max(np.abs(lit.state)):.0f}, max |y| {np.max(np.abs(lit.y)):.0f}: state "
+          f"{hs.rel_err(st, lit.state):.2e} rel, outputs {hs.rel_err(out, lit.out):.2e} normwise")
+    assert np.all(np.isfinite(st)) and hs.rel_err(st, lit.state) <= STATE_TOL
+    assert hs.rel_err(out, lit.out) <= OUT_REL
+    # small: |S| and |v| of 1e-5
+    small = o.Rows(heads, t, rows.qkv.copy(), rows.a, rows.b, rows.gate)
+    qkv = small.qkv.reshape(t, 3, heads * DK)
+    qkv[:, 2] = o.bf16_round(qkv[:, 2] * 2.0 ** -17)
+    conv_small = conv.copy().reshape(WINDOW, 3, heads * DK)
+    conv_small[:, 2] = o.bf16_round(conv_small[:, 2] * 2.0 ** -17)
+    s_small = o.synth_state(heads, 7702, 1e-5)
+    out, st, _ = hs.prefill_gpu(p, conv_small.reshape(-1), s_small, small)
+    lit = o.literal_chain(p, conv_small.reshape(-1), s_small, small, threads=8)
+    print(f"small: max |S| {np.max(np.abs(lit.state)):.1e}: state max-abs {hs.max_abs(st, lit.state):.1e} "
+          f"({hs.rel_err(st, lit.state):.1e} rel)")
+    assert hs.max_abs(st, lit.state) <= 1e-7
+    # beyond: 4 |S| does not fit fp16
+    s_far = o.synth_state(heads, 7703, 60000.0)
+    _, st, _ = hs.prefill_gpu(p, conv, s_far, rows)
+    lit = o.literal_chain(p, conv, s_far, rows, threads=8)
+    assert np.all(np.isfinite(lit.state))
+    print(f"beyond: {int((~np.isfinite(st)).sum())} of {st.size} state elements are not finite")
+    assert not np.all(np.isfinite(st))
