@@ -139,11 +139,11 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
         __syncthreads();
         if (!live) continue;
         while (k0 < pw) {                         // in pairs, so that the two register sets are compile-time choices
-            request(wb, k0 + STEP * UNROLL);
+            if (M <= 4 || k0 + STEP * UNROLL < pw) request(wb, k0 + STEP * UNROLL);   // (short pieces: no loads past the end)
             work(wa, k0);
             k0 += STEP * UNROLL;
             if (k0 >= pw) break;
-            request(wa, k0 + STEP * UNROLL);
+            if (M <= 4 || k0 + STEP * UNROLL < pw) request(wa, k0 + STEP * UNROLL);
             work(wb, k0);
             k0 += STEP * UNROLL;
         }
@@ -320,8 +320,9 @@ int32_t launch_mo(const uint16_t* x, long long ldx, long long x_gs, const uint16
                   long long o_gs, hipStream_t stream) {
     const int kc = k / ksplit;
     // the widest piece of the K range whose activations fit 32 KiB (64 KiB for one row: no second piece up to
-    // k = 16,384), a multiple of 256: more workgroups per CU matter more than fewer barriers
-    int kp = (M == 1 ? LDS_BYTES : LDS_BYTES / 2) / (4 * M) / STEP * STEP;
+    // k = 16,384; and from five rows up, where a 32 KiB piece would be shorter than the steps requested together
+    // and every piece's first loads wait behind a barrier: o_proj with eight rows 34.7 -> 31.6 us), a multiple of 256
+    int kp = (M == 1 || M > 4 ? LDS_BYTES : LDS_BYTES / 2) / (4 * M) / STEP * STEP;
     if (kp > kc) kp = kc;
     const size_t lds = (size_t)M * kp * 4;
     const int block_outs = (THREADS / 32) * OUTS;

@@ -291,6 +291,15 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // otherwise the per-lane addresses of the body are hoisted out of the chunk loop and spill.
     asm volatile("" : "+v"(t));
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63;
+    // Two workgroups share a CU, a wave of each on every SIMD, and the SIMD issues for the older wave first: left
+    // alone, the workgroup that arrived first runs its chunks at full speed (23 us), the other fills the gaps (44 us)
+    // and then finishes alone with nothing to hide its waits behind. So the waves' priority alternates from chunk to
+    // chunk, the other way round in the second workgroup of a CU (workgroups fill the 256 CUs in the order of their
+    // index), which keeps the two level and their phases apart: 66.4 -> 60.5 us per pass of 1024 rows. (Raising the
+    // priority of the short phases between barriers on top of this took 3 us of that back.)
+    __builtin_amdgcn_s_setprio(0);
+    if ((((c - c_first) ^ (((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) >> 8)) & 1) != 0)
+        __builtin_amdgcn_s_setprio(1);
     const int i = lane & 15, g = lane >> 4;       // this lane's row of the sub-chunk and its set of 32 channels
     // what the lane holds after a transpose16: position cl_t (of the sixteen values the four lanes of a row put in:
     // lane group cl_t / 4, its value cl_t % 4) of rows rl_t .. rl_t + 3 of the sub-chunk
@@ -429,10 +438,6 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         beta_s[t] = t < n ? bfround(fast_sigmoid(bf2f(b_raw))) : 0.0f;
     }
     __syncthreads();
-    // From here to the end of the chunk the phases are short and end in barriers, except for the operands: a wave in
-    // them goes ahead of the other workgroup's wave on its SIMD, which is most likely in a long elementwise phase
-    // and loses nothing by waiting a few instructions.
-    __builtin_amdgcn_s_setprio(2);
     // v leaves for the workspace ([value][row], as the inter pass adds it to its accumulators): its place in LDS
     // is taken by the diagonal blocks after the next barrier
 #pragma unroll
@@ -473,7 +478,6 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     }
 
     __syncthreads();                              // the factors are in place, v has left
-    __builtin_amdgcn_s_setprio(0);
 
     // ---- operands. Per element: ep = e^{G_i - G_0} and its reciprocal (G_0: the sub-chunk's first row, so that
     // fifteen rows of decay bound the exponent); e^{G_15 - G_i} is the last row's ep over the own one.
@@ -581,7 +585,6 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         put_M(accM, wave, wave);
     }
     __syncthreads();                              // the column operands of every sub-chunk are in place
-    __builtin_amdgcn_s_setprio(2);
     uint16_t* TT = reinterpret_cast<uint16_t*>(smem + I_TT);
     if (wave == 0) {
         // Sub-chunk 0 has no tiles left of its diagonal, so while the other waves compute theirs wave 0 does what
@@ -727,7 +730,6 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         }
     }
     __syncthreads();                              // the next chunk's conv writes VT before its first barrier
-    __builtin_amdgcn_s_setprio(0);
     }
 }
 

@@ -170,8 +170,9 @@ int glm53f_kda_conv_shift_batch(int32_t channels, int32_t layers, int32_t batch,
 
 /**
  * Bytes of workspace for the prefill to run `rows_per_pass` rows of every request per pass; 0 on bad
- * arguments. On this build a chunk is 64 rows and costs 74,240 bytes per head and request. Replaces
- * glm53f_kda_prefill_workspace_bytes (header :204, kda_prefill.cu:695-698; 34,816 bytes per 16 rows there).
+ * arguments. On this build a chunk is 64 rows and costs 147,968 bytes per head and request (every operand of the
+ * state-carrying pass as a pair of fp16 planes). Replaces glm53f_kda_prefill_workspace_bytes (header :204,
+ * kda_prefill.cu:695-698; 34,816 bytes per 16 rows there).
  */
 int64_t glm53f_kda_prefill_workspace_bytes(int32_t heads, int32_t batch, int32_t rows_per_pass);
 
@@ -180,11 +181,20 @@ int64_t glm53f_kda_prefill_workspace_bytes(int32_t heads, int32_t batch, int32_t
  * through the chunked (WY/UT) form of the delta rule on the matrix cores. Inputs and outputs as
  * glm53f_kda_chain without replay inputs; the conv window is advanced past the rows in place.
  * state_out must not be NULL (it may equal state_in). lower must lie in [-5.8, 0].
- * value_blocks: 0 (choose), 1, 2 or 4 workgroups per head in the state-carrying pass.
- * workspace: at least glm53f_kda_prefill_workspace_bytes(heads, 1, 64) bytes; its size sets the rows per
- * pass. Results agree with the chain within bf16-output / 1e-3-state tolerance, not bit for bit; they do
- * not depend on the workspace size or on how requests are batched. Replaces glm53f_kda_prefill
- * (header :223-232, kda_prefill.cu:700-710).
+ * value_blocks: 0, 1, 2 or 4 are accepted as the reference accepts them (anything else is rejected) and have no
+ * effect: this build always runs four workgroups of 32 value columns per head in the state-carrying pass.
+ * workspace: at least glm53f_kda_prefill_workspace_bytes(heads, 1, 64) bytes; its size bounds the rows per
+ * pass (the library may use less of it: passes are cut to what the 256 MB cache behind the L2 holds).
+ * Numerics: every matrix-core operand is a pair of fp16 values (22 significant bits), accumulation is f32.
+ * Against the chain: f32 states agree to about 1e-6 normwise (1e-4 where decay is slow enough that thousands of
+ * rows are remembered) and about 0.05 % of the bf16 outputs fall on the other side of a rounding boundary; not bit
+ * for bit. Results do not depend on the workspace size or on how requests are batched.
+ * Domain: the state, V - Kd S and V' pass through fp16 with scale 4, so the 2-norm of a value row of the state
+ * (its 128 keys) plus |v| must stay below 16,376 - states below 1,400 in magnitude always do - and those three carry
+ * an absolute error floor of 7.5e-9. Beyond that the state comes out non-finite where the f32 recurrence (and
+ * glm53f_kda_chain) stays finite. The device arrays are not inspected on the host.
+ * The first call on a device also sets two kernel attributes (LDS above 64 KiB) under a lock; make one call on
+ * each device before capturing a stream. Replaces glm53f_kda_prefill (header :223-232, kda_prefill.cu:700-710).
  */
 int glm53f_kda_prefill(int32_t heads, int32_t rows, const glm53f_bf16* p, int64_t p_stride, int64_t b_off,
     const glm53f_bf16* a, int64_t a_stride, const glm53f_bf16* g, int64_t g_stride, glm53f_bf16* conv,
