@@ -84,7 +84,6 @@ __device__ __forceinline__ f32x4 mfma_f16(uint4 a, uint4 b, f32x4 c) {
 // LDS map of intra_kernel, bytes. 76.5 KB: two workgroups share a CU.
 constexpr int LDD = SUB + 4;                      // f32 row stride of a diagonal block of L (16-byte multiple)
 constexpr int LDT = 40, LDZ = 24;                 // 16-bit row strides of TT and Z (16-byte multiples)
-constexpr int LDK = DK + 4;                       // f32 row stride of the column operands
 constexpr int NFAC = 14;                          // per-channel factors between sub-chunks (see factor_index)
 constexpr int I_CW = 0;                           // u32 [q | k | v][128 channels][4 taps]: the head's conv weights
 constexpr int I_DTB = I_CW + 3 * DK * TAPS * 4;   // f32 [128]: the head's dt_bias, times -rate log2(e)
@@ -96,12 +95,13 @@ constexpr int I_TT = I_LD + 4 * SUB * LDD * 4;    //   and fp16 x 2 [64][LDT]: r
 constexpr int TT_PLANE = CH * LDT;                //   (elements from the hi plane to the lo plane)
 constexpr int I_LN = I_VT + DV * LD64 * 2;        // fp16 x 2 [64][LD64]: -L below the block diagonal, zero elsewhere
 constexpr int LN_PLANE = CH * LD64;
-constexpr int I_KCE = I_LN + 2 * CH * LD64 * 2;   // f32 [3][16][LDK]: k e^{G_end - G} of sub-chunks 0..2, row major;
+constexpr int I_KCE = I_LN + 2 * CH * LD64 * 2;   // fp16 x 2 [3][16][LD128]: 2^14 k e^{G_end - G} of sub-chunks 0..2, row major;
+constexpr int KC_PLANE = 3 * SUB * LD128;         //   (elements from the hi plane to the lo plane)
 constexpr int I_RT = I_KCE;                       //   later fp16 x 2 [64 columns][LD64]: the solve's right-hand sides,
 constexpr int RT_PLANE = CH * LD64;               //   transposed,
 constexpr int I_Z = I_RT + 2 * CH * LD64 * 2;     //   and fp16 x 2 [4 column tiles][16][LDZ]: a tile of Z on its way back
 constexpr int Z_PLANE = 4 * SUB * LDZ;
-constexpr int I_FAC = I_KCE + 3 * SUB * LDK * 4;  // f32 [NFAC][128]
+constexpr int I_FAC = I_KCE + 2 * KC_PLANE * 2;    // f32 [NFAC][128]
 constexpr int INTRA_LDS = I_FAC + NFAC * DK * 4;
 constexpr int INTRA_CPW = 2;                      // consecutive chunks of a head per intra workgroup
 static_assert(I_TT + 2 * CH * LDT * 2 <= I_LN, "the diagonal blocks and TT fit where v was");
@@ -253,7 +253,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     uint16_t* VT = reinterpret_cast<uint16_t*>(smem + I_VT);
     uint16_t* Ln = reinterpret_cast<uint16_t*>(smem + I_LN);
     float* Ld = reinterpret_cast<float*>(smem + I_LD);
-    float* KcE = reinterpret_cast<float*>(smem + I_KCE);
+    uint16_t* KcE = reinterpret_cast<uint16_t*>(smem + I_KCE);
     float* fac = reinterpret_cast<float*>(smem + I_FAC);
     float* first = reinterpret_cast<float*>(smem + I_KCE);          // [4][128]: until the column operands go there
 
@@ -468,12 +468,12 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         } else {
             fac[6 * DK + d] = SC_K * __builtin_amdgcn_exp2f(t3);
             fac[7 * DK + d] = SC_K;
-            fac[factor_index(1, 0) * DK + d] = __builtin_amdgcn_exp2f(u1);
-            fac[factor_index(2, 0) * DK + d] = __builtin_amdgcn_exp2f(t1 + u2);
-            fac[factor_index(2, 1) * DK + d] = __builtin_amdgcn_exp2f(u2);
-            fac[factor_index(3, 0) * DK + d] = __builtin_amdgcn_exp2f(t1 + t2 + u3);
-            fac[factor_index(3, 1) * DK + d] = __builtin_amdgcn_exp2f(t2 + u3);
-            fac[factor_index(3, 2) * DK + d] = __builtin_amdgcn_exp2f(u3);
+            fac[factor_index(1, 0) * DK + d] = SC_K * __builtin_amdgcn_exp2f(u1);
+            fac[factor_index(2, 0) * DK + d] = SC_K * __builtin_amdgcn_exp2f(t1 + u2);
+            fac[factor_index(2, 1) * DK + d] = SC_K * __builtin_amdgcn_exp2f(u2);
+            fac[factor_index(3, 0) * DK + d] = SC_K * __builtin_amdgcn_exp2f(t1 + t2 + u3);
+            fac[factor_index(3, 1) * DK + d] = SC_K * __builtin_amdgcn_exp2f(t2 + u3);
+            fac[factor_index(3, 2) * DK + d] = SC_K * __builtin_amdgcn_exp2f(u3);
         }
     }
 
@@ -491,7 +491,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // Store a finished tile at block (rb, cb). L = beta_i * acc: a diagonal block (strictly lower) in f32 for the
     // inversion, a block below the diagonal negated as an fp16 pair, an MFMA operand of the block solve. M (lower
     // with the diagonal; acc holds 8 M) goes to the workspace.
-    auto put_L = [&](f32x4 acc, int rb, int cb) {
+    auto put_L = [&](f32x4 acc, int rb, int cb, float unit) {
         const int gi = SUB * rb + cl, gj = SUB * cb + rl;
         const float bi = beta_s[gi];
         if (rb == cb) {
@@ -503,16 +503,16 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             *reinterpret_cast<uint2*>(Ln + LN_PLANE + gi * LD64 + gj) = make_uint2(0u, 0u);
         } else {
             uint2 hi, lo;
-            split_h4(scaled(acc, -SC_K * bi), hi, lo);
+            split_h4(scaled(acc, -SC_K * unit * bi), hi, lo);
             *reinterpret_cast<uint2*>(Ln + gi * LD64 + gj) = hi;
             *reinterpret_cast<uint2*>(Ln + LN_PLANE + gi * LD64 + gj) = lo;
         }
     };
-    auto put_M = [&](f32x4 acc, int rb, int cb) {
+    auto put_M = [&](f32x4 acc, int rb, int cb, float unit) {
         const int gi = SUB * rb + cl, gj = SUB * cb + rl;
         f32x4 v;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = (rb != cb || gj + r <= gi) ? acc[r] * SC_K : 0.0f;
+        for (int r = 0; r < 4; ++r) v[r] = (rb != cb || gj + r <= gi) ? acc[r] * (SC_K * unit) : 0.0f;
         uint2 hi, lo;
         split_h4(v, hi, lo);
         *reinterpret_cast<uint2*>(Mg + panel_index(CH, gi, gj)) = hi;
@@ -576,13 +576,18 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 *reinterpret_cast<u32x4*>(dst + PLANE16) = lo;
             }
             if (wave < 3) {
-                float* dst = KcE + (wave * SUB + i) * LDK + 32 * p + 8 * g;
-                *reinterpret_cast<f32x4*>(dst) = f32x4{kc[0], kc[1], kc[2], kc[3]};
-                *reinterpret_cast<f32x4*>(dst + 4) = f32x4{kc[4], kc[5], kc[6], kc[7]};
+                float kcs[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) kcs[e] = kc[e] * SC_K;
+                u32x4 hi, lo;
+                split_h8(kcs, hi, lo);
+                uint16_t* dst = KcE + (wave * SUB + i) * LD128 + 32 * p + 8 * g;
+                *reinterpret_cast<u32x4*>(dst) = hi;
+                *reinterpret_cast<u32x4*>(dst + KC_PLANE) = lo;
             }
         }
-        put_L(accL, wave, wave);
-        put_M(accM, wave, wave);
+        put_L(accL, wave, wave, 1.0f);
+        put_M(accM, wave, wave, 1.0f);
     }
     __syncthreads();                              // the column operands of every sub-chunk are in place
     uint16_t* TT = reinterpret_cast<uint16_t*>(smem + I_TT);
@@ -637,28 +642,35 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             row[TT_PLANE + SUB + j] = f2h(tn - h2f(tnh));
         }
     } else {
-        // tiles left of the diagonal: rows of sub-chunk `wave` against the columns of sub-chunk cb, on the f32
-        // matrix instruction. In step (s, e) lane group g supplies channel 32 s + 8 g + e on both sides (which k a
-        // lane supplies is free as long as both operands agree).
+        // tiles left of the diagonal: rows of sub-chunk `wave` against the columns of sub-chunk cb. Both sides have
+        // exponents <= 0 here (the column side relative to its sub-chunk's end, the row side with the decay between
+        // the sub-chunks in its factor), so they fit fp16 pairs with scale 2^14 and the tiles take the fp16 matrix
+        // instruction: 24 of 16 cycles per pair of tiles instead of 64 of 32 on the f32 one, for the cost of
+        // splitting the row side once per column block. In step p lane group g supplies channels 32 p + 8 g .. + 7
+        // on both sides; the accumulators are in units of 2^28.
 #pragma unroll 1
         for (int cb = 0; cb < wave; ++cb) {
             const float* df = fac + factor_index(wave, cb) * DK + 8 * g;
-            const float* kcol = KcE + (cb * SUB + i) * LDK + 8 * g;
             f32x4 accL = zero, accM = zero;
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const f32x4 d0 = *reinterpret_cast<const f32x4*>(df + 32 * s), d1 = *reinterpret_cast<const f32x4*>(df + 32 * s + 4);
-                const f32x4 c0 = *reinterpret_cast<const f32x4*>(kcol + 32 * s), c1 = *reinterpret_cast<const f32x4*>(kcol + 32 * s + 4);
+            for (int p = 0; p < 4; ++p) {
+                const f32x4 d0 = *reinterpret_cast<const f32x4*>(df + 32 * p), d1 = *reinterpret_cast<const f32x4*>(df + 32 * p + 4);
+                float rk[8], rq[8];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float f = e < 4 ? d0[e] : d1[e - 4];
-                    const float col = e < 4 ? c0[e] : c1[e - 4];
-                    accL = __builtin_amdgcn_mfma_f32_16x16x4f32(col, kep[8 * s + e] * f, accL, 0, 0, 0);
-                    accM = __builtin_amdgcn_mfma_f32_16x16x4f32(col, qep[8 * s + e] * f, accM, 0, 0, 0);
+                    rk[e] = kep[8 * p + e] * f;
+                    rq[e] = qep[8 * p + e] * f;
                 }
+                u32x4 kh, kl, qh, ql;
+                split_h8(rk, kh, kl);
+                split_h8(rq, qh, ql);
+                const uint4 ch = frag(KcE, LD128, cb * SUB, 32 * p, lane), cl2 = frag(KcE + KC_PLANE, LD128, cb * SUB, 32 * p, lane);
+                accL = mfma_hl(ch, cl2, make_uint4(kh[0], kh[1], kh[2], kh[3]), make_uint4(kl[0], kl[1], kl[2], kl[3]), accL);
+                accM = mfma_hl(ch, cl2, make_uint4(qh[0], qh[1], qh[2], qh[3]), make_uint4(ql[0], ql[1], ql[2], ql[3]), accM);
             }
-            put_L(accL, wave, cb);
-            put_M(accM, wave, cb);
+            put_L(accL, wave, cb, 1.0f / (SC_K * SC_K));
+            put_M(accM, wave, cb, 1.0f / (SC_K * SC_K));
         }
     }
     __syncthreads();                              // L and TT are complete; the factors and column operands are dead
