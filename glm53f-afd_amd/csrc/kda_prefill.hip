@@ -145,6 +145,9 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
 }
 
 // The same without an addend, in the three-operand encoding: a sum that starts here needs no zeroed accumulator.
+// (The one inline assembly of this file, and register operands only. An assembly *load* has no place here: the
+// compiler does not know that its destination is still in flight, moves or reuses the register, and the data lands
+// on whatever lives there by then - an address, once, which faults the GPU.)
 __device__ __forceinline__ float dot2_bf16_first(uint32_t a, uint32_t b) {
     float r;
     asm("v_dot2_f32_bf16 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(b));
@@ -1292,6 +1295,8 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
 }  // namespace kda
 
 using namespace kda;
+
+extern "C" int glm53f_kda_init(void) { return allow_large_lds(); }
 
 extern "C" int64_t glm53f_kda_prefill_workspace_bytes(int32_t heads, int32_t batch, int32_t rows_per_pass) {
     if (heads < 1 || batch < 1 || rows_per_pass < 1) return 0;

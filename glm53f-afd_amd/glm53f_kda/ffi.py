@@ -42,6 +42,7 @@ PROTOTYPES = {
     "glm53f_kda_chain_shift_batch_bf16state": (C.c_int, [i32, i32, ptr] + _ROWS + [ptr, ptr, ptr, ptr, ptr, ptr]
                                                + _WEIGHTS + [ptr, i64] + _SAVES + [ptr]),
     "glm53f_kda_arch": (C.c_char_p, []),
+    "glm53f_kda_init": (C.c_int, []),
 }
 
 # The 13 entry points of the reference's ABI (crates/glm53f-kda/tests/provenance.rs:41-69).

@@ -290,6 +290,16 @@ int glm53f_kda_chain_shift_batch_bf16state(int32_t heads, int32_t batch, const i
 /** The gfx architecture the kernels were compiled for ("gfx950"). */
 const char* glm53f_kda_arch(void);
 
+/**
+ * Per-device set-up of the current device, once: the prefill kernels ask for more than 64 KiB of LDS, which is an
+ * attribute of each device's copy of a kernel. Every prefill entry point does the same on its first call on a
+ * device (under a lock), so calling this is only needed where that first call would come at a bad time: inside a
+ * stream capture, or from two host threads that must not wait for each other. Launches nothing, allocates nothing;
+ * returns 0 or the runtime's error code. No counterpart in the reference (its kernels stay under 48 KiB of shared
+ * memory).
+ */
+int glm53f_kda_init(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,7 +26,7 @@ def test_header_declares_the_reference_entry_points():
     assert len(ffi.REFERENCE_SYMBOLS) == 13
     extra = set(decl) - set(ffi.REFERENCE_SYMBOLS)
     assert extra == {"glm53f_kda_verify_batch_bf16state", "glm53f_kda_select_batch_bf16state", "glm53f_kda_arch",
-                     "glm53f_kda_chain_shift_batch", "glm53f_kda_chain_shift_batch_bf16state"}
+                     "glm53f_kda_chain_shift_batch", "glm53f_kda_chain_shift_batch_bf16state", "glm53f_kda_init"}
 
 
 def test_library_exports_every_declared_symbol():
