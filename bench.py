@@ -34,18 +34,19 @@ from glm53f_kda import DK, DV, HEADS, LAYERS, WINDOW, channels, ffi, state_len
 # script's legs, scaled by the same counters over the 1 GiB copy of --only copy: x2.00 and x1.00). Measured
 # offline; the summaries are kept in profiles/.
 TRAFFIC_BYTES = {
-    "decode_chain": (36_794 + 33_024) * 1024,            # per plain chain launch, 16 slots x 1 row
-    "verify_chain": (167_880 + 1_585_201) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
-    "prefill_2048_rows": (152_067 + 148_534 + 148_598 + 36_866 + 65_741 + 32_912) * 1024,   # intra, inter, norm: read + written
-    "mark_state_pages": (69_930 + 70_852) * 1024,
-    "gemv_kda_proj_1row": (197_885 + 48) * 1024,         # per launch: the weights once, the activations, the outputs
+    "decode_chain": (36_798 + 33_024) * 1024,            # per plain chain launch, 16 slots x 1 row
+    "verify_chain": (167_883 + 1_585_724) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
+    # two passes of 1024 rows (intra read + written, inter read + written) and one norm launch
+    "prefill_2048_rows": (2 * (74_088 + 148_951 + 144_086 + 20_483) + 65_755 + 32_912) * 1024,
+    "mark_state_pages": (69_926 + 70_840) * 1024,
+    "gemv_kda_proj_1row": (197_891 + 48) * 1024,         # per launch: the weights once, the activations, the outputs
 }
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
 DEV = "cuda:0"
 
 METRIC = "KDA prefill tok/s per layer at T=8K (MFMA %); decode state GB/s at 16 slots"
-PREFILL_DTYPE = "fp16 MFMA operands, f32 accumulate"
+PREFILL_DTYPE = "fp16 hi/lo operand pairs on the MFMA (f32-class products), f32 accumulate"
 
 
 def ptr(t, off=0):
@@ -269,7 +270,7 @@ def bench_prefill(steps, warmup, stream, cpu=True):
         "tok_per_s_per_layer": total / (ms * 1e-3), "ms_per_8192_tokens": ms,
         "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": TRAFFIC_BYTES["prefill_2048_rows"], "traffic_unit": "B per 2048-row call (3 kernels)",
+                     "traffic": TRAFFIC_BYTES["prefill_2048_rows"], "traffic_unit": "B per 2048-row call (2 intra + 2 inter launches of 1024 rows, 1 norm launch)",
                      "kernel": "prefill (intra + inter + norm with the conv window advance, whole call)",
                      "flops_per_token": 11_709_099, "hbm_GBps_compulsory": io_bytes / (ms * 1e-3) / 1e9,
                      "hbm_frac": io_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
