@@ -190,6 +190,146 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
     }
 }
 
+// The same contract for five to eight rows when the wide kernel below would leave CUs without a workgroup (the output
+// projection: n = 4096). The two halves of a wave take the same two outputs and split the rows between them (their
+// loads of a weight piece name the same address: one fetch), so a lane carries a quarter of the accumulators of two
+// outputs x eight rows, the rows' activations are read from LDS once for two outputs, and there are waves enough to
+// keep two workgroups on every CU. The weight stream does not stop at the pieces of the K range: a group of four
+// steps is always in flight while the other is worked on, and the next piece's activations are requested before
+// the current piece is worked on. Each accumulator still sees its products in the model's order.
+constexpr int SPLIT_OUTS = 2, SPLIT_UNROLL = 4;
+constexpr int SPLIT_BLOCK_OUTS = (THREADS / 64) * SPLIT_OUTS;        // 8: one counter per workgroup
+constexpr int SPLIT_KP = 2 * STEP * SPLIT_UNROLL;                    // 2048: a piece is two groups of steps
+
+template <int M, bool F32>
+__global__ void __launch_bounds__(THREADS) gemv_split_rows_kernel(const uint16_t* __restrict__ x, long long ldx,
+                                                                  long long x_gs, const uint16_t* __restrict__ w,
+                                                                  long long ldw, long long w_gs, int n, int kc,
+                                                                  float* __restrict__ partials,
+                                                                  unsigned* __restrict__ sync, void* __restrict__ out,
+                                                                  long long ldo, long long o_gs) {
+    constexpr int MR = (M + 1) / 2;                                   // rows of a lane: row0 .. row0 + MR - 1, below M
+    constexpr int kp = SPLIT_KP, GROUP = STEP * SPLIT_UNROLL;
+    static_assert(M * kp * 4 <= LDS_BYTES, "a piece's activations fit the LDS of a launch without an attribute");
+    __shared__ __align__(16) float xs[M * kp];
+    const int t = threadIdx.x, l = t & 31;
+    const int row0 = ((t >> 5) & 1) * MR;
+    const int g = blockIdx.z, split = blockIdx.y, nsplit = gridDim.y;
+    const int o0 = blockIdx.x * SPLIT_BLOCK_OUTS + (t >> 6) * SPLIT_OUTS;   // n % 8 == 0: all eight exist
+    const int lo = split * kc;
+    const uint16_t* xg = x + g * x_gs + lo;
+    const uint16_t* w0 = w + g * w_gs + (long long)o0 * ldw + lo;
+
+    float acc[SPLIT_OUTS][MR];
+#pragma unroll
+    for (int r = 0; r < SPLIT_OUTS; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[r][m] = 0.0f;
+
+    // lane l takes k = 8 l + 256 i while that is below kc; kq: the first k of a group of steps
+    auto request = [&](u32x4 (&wv)[SPLIT_UNROLL][SPLIT_OUTS], int kq) {
+#pragma unroll
+        for (int u = 0; u < SPLIT_UNROLL; ++u)
+#pragma unroll
+            for (int r = 0; r < SPLIT_OUTS; ++r)   // unconditional (a step past the range re-reads its last piece)
+                wv[u][r] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x4*>(w0 + r * ldw + min(kq + 8 * l + STEP * u, kc - 8)));
+    };
+    // p0: the first k of the staged piece
+    auto work = [&](const u32x4 (&wv)[SPLIT_UNROLL][SPLIT_OUTS], int kq, int p0) {
+#pragma unroll
+        for (int u = 0; u < SPLIT_UNROLL; ++u) {
+            const int k = kq + 8 * l + STEP * u;
+            if (k >= kc) break;
+            float wf[SPLIT_OUTS][8];
+#pragma unroll
+            for (int r = 0; r < SPLIT_OUTS; ++r)
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    wf[r][2 * d] = lo16(wv[u][r][d]);
+                    wf[r][2 * d + 1] = hi16(wv[u][r][d]);
+                }
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                if (2 * MR != M && m == MR - 1 && row0 != 0) break;   // an odd M: the second half is one row short
+                // a step's 256 values sit as the 32 lanes' first four, then their second four: the lanes of a half
+                // read consecutive 16-byte pieces (lane-major, 32 bytes apart, they would meet in the banks)
+                const f32x4* xp = reinterpret_cast<const f32x4*>(xs + (row0 + m) * kp + (k - p0) - 4 * l);
+                const f32x4 xa = xp[0], xb = xp[32];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float xv = j < 4 ? xa[j] : xb[j - 4];
+#pragma unroll
+                    for (int r = 0; r < SPLIT_OUTS; ++r) acc[r][m] = __builtin_fmaf(xv, wf[r][j], acc[r][m]);
+                }
+            }
+        }
+    };
+    // A piece's activations: lane t takes the eight values at k = p0 + 8 t of every row (kp = 8 x 256 lanes).
+    u32x4 xq[M];
+    auto request_x = [&](int p0) {
+        const int k = min(p0 + 8 * t, kc - 8);
+#pragma unroll
+        for (int m = 0; m < M; ++m) xq[m] = *reinterpret_cast<const u32x4*>(xg + m * ldx + k);
+    };
+    auto stage_x = [&]() {
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            f32x4* dst = reinterpret_cast<f32x4*>(xs + m * kp + 8 * t - 4 * (t & 31));
+            dst[0] = f32x4{lo16(xq[m][0]), hi16(xq[m][0]), lo16(xq[m][1]), hi16(xq[m][1])};
+            dst[32] = f32x4{lo16(xq[m][2]), hi16(xq[m][2]), lo16(xq[m][3]), hi16(xq[m][3])};
+        }
+    };
+
+    u32x4 wa[SPLIT_UNROLL][SPLIT_OUTS], wb[SPLIT_UNROLL][SPLIT_OUTS];
+    request(wa, 0);
+    request_x(0);
+    for (int p0 = 0; p0 < kc; p0 += kp) {
+        if (p0 > 0) __syncthreads();              // every lane is past its reads of the piece before
+        stage_x();
+        __syncthreads();
+        request(wb, p0 + GROUP);
+        if (p0 + kp < kc) request_x(p0 + kp);
+        work(wa, p0, p0);
+        request(wa, p0 + kp);
+        if (p0 + GROUP < kc) work(wb, p0 + GROUP, p0);
+    }
+
+    void* og = F32 ? static_cast<void*>(static_cast<float*>(out) + g * o_gs)
+                   : static_cast<void*>(static_cast<uint16_t*>(out) + g * o_gs);
+#pragma unroll
+    for (int r = 0; r < SPLIT_OUTS; ++r)
+#pragma unroll
+        for (int mi = 0; mi < MR; ++mi) {
+            const float v = half_wave_sum(acc[r][mi]);
+            const int m = row0 + mi;
+            if (m < M && l == ((r * MR + mi) & 31)) {
+                if (nsplit > 1) partials[(((long long)g * nsplit + split) * M + m) * n + o0 + r] = v;
+                else store_out<F32>(og, (long long)m * ldo + o0 + r, v);
+            }
+        }
+    if (nsplit == 1) return;
+
+    int& last = *reinterpret_cast<int*>(xs);      // as above: the last workgroup of these eight outputs adds the splits
+    __threadfence();
+    __syncthreads();
+    unsigned* counter = sync + (long long)g * (n / 8) + blockIdx.x;
+    if (t == 0) last = atomicAdd(counter, 1u) == (unsigned)(nsplit - 1);
+    __syncthreads();
+    if (!last) return;
+    __threadfence();
+    if (t == 0) *counter = 0;
+    const long long split_stride = (long long)M * n;
+    for (int e = t; e < SPLIT_BLOCK_OUTS * M; e += THREADS) {
+        const int m = e / SPLIT_BLOCK_OUTS, o = blockIdx.x * SPLIT_BLOCK_OUTS + e % SPLIT_BLOCK_OUTS;
+        const long long base = ((long long)g * nsplit * M + m) * n + o;
+        float s = __hip_atomic_load(partials + base, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int kk = 1; kk < nsplit; ++kk)
+            s = s + __hip_atomic_load(partials + base + kk * split_stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        store_out<F32>(og, (long long)m * ldo + o, s);
+    }
+}
+
 // The same contract for three rows and more, where a lane's arithmetic (rows x 8 fused multiply-adds per weight
 // word pair) and its reads of the activations weigh as much as the weight stream: half a wave owns eight outputs
 // and walks the K steps in the outer loop, so that the rows' activations of a step are read from LDS once for all
@@ -350,9 +490,16 @@ int32_t launch_m(const uint16_t* x, long long ldx, long long x_gs, const uint16_
                                                                                      partials, sync, out, ldo, o_gs);
         return (int32_t)hipGetLastError();
     }
-    if (n % 16 == 0 && blocks8 >= 2 * 1024)
-        return launch_mo<M, 2, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
-    return launch_mo<M, 1, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+    if constexpr (M > 4) {
+        const dim3 grid((unsigned)(n / SPLIT_BLOCK_OUTS), (unsigned)ksplit, (unsigned)groups);
+        gemv_split_rows_kernel<M, F32><<<grid, THREADS, 0, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, k / ksplit, partials,
+                                                                     sync, out, ldo, o_gs);
+        return (int32_t)hipGetLastError();
+    } else {
+        if (n % 16 == 0 && blocks8 >= 2 * 1024)
+            return launch_mo<M, 2, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+        return launch_mo<M, 1, F32>(x, ldx, x_gs, w, ldw, w_gs, groups, n, k, ksplit, partials, sync, out, ldo, o_gs, stream);
+    }
 }
 
 template <bool F32>

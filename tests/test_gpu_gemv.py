@@ -198,3 +198,20 @@ def test_engine_dispatch_and_the_vendor_gemm_within_rounding():
         Gemm(GemmPolicy(gemv_max_rows=9))
     with pytest.raises(GemmError):                                    # the launcher's own checks surface as errors
         gemm.gemv(x.data_ptr() + 2, k, 0, mat, 8, out.data_ptr(), n, 0, False)
+
+
+def test_gemv_output_projection_shape_with_five_to_eight_rows():
+    """The output projection under a verify window: 8192 -> 4096 without a K split, five to eight rows (the kernel
+    whose wave halves split the rows), against the model on a sample of the outputs."""
+    sc = Scratch()
+    rng = np.random.default_rng(8)
+    n, k = 4096, 8192
+    w = bf16_normal(rng, (1, n, k), 0.02)
+    x = bf16_normal(rng, (1, 8, k), 1.0)
+    assert fwd.glm53f_fwd_gemv_ksplit(1, n, k) == 1
+    sample = rng.permutation(n)[:512]
+    for f32_out in (False, True):
+        want = model(x, w[:, sample], 8, 1, f32_out)
+        for rows in (5, 6, 7, 8):
+            got = run(sc, x, w, rows, 1, f32_out)
+            assert np.array_equal(got[:, :, sample].view(np.uint32), want[:, :rows].view(np.uint32)), (rows, f32_out)
