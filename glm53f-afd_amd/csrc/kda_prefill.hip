@@ -597,18 +597,19 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     if (wave == 0) {
         // Sub-chunk 0 has no tiles left of its diagonal, so while the other waves compute theirs wave 0 does what
         // needs the diagonal blocks only.
-        // M and -L above the block diagonal are zero: blocks (0,1), (0,2), (0,3), (1,2), (1,3), (2,3), in 128-bit
-        // pieces (two per row of a block), both planes
-#pragma unroll
-        for (int it = 0; it < 3; ++it) {
-            const int e = lane + 64 * it, blk = e >> 5, r = (e >> 1) & 15, half = e & 1;
-            const int rb = blk < 3 ? 0 : (blk < 5 ? 1 : 2);
-            const int cb = blk < 3 ? blk + 1 : (blk < 5 ? blk - 1 : 3);
+        // M and T' are zero above the block diagonal. The inter pass reads a row's columns 0..31 always and 32..63
+        // from row 32 on, so of the six blocks there it meets two, (0,1) and (2,3): those are written as zeros, in
+        // 128-bit pieces (two per row of a block), both planes; the other four stay as they are, unread. (-L above the
+        // diagonal is never read either: the solve below starts a block column at its diagonal block.)
+        {
+            const int blk = lane >> 5, r = (lane >> 1) & 15, half = lane & 1;
+            const int rb = 2 * blk, cb = 2 * blk + 1;
             const u32x4 z = {0u, 0u, 0u, 0u};
+            uint16_t* Tz = reinterpret_cast<uint16_t*>(wsc + WS_TP);
             *reinterpret_cast<u32x4*>(Mg + panel_index(CH, SUB * rb + r, SUB * cb + 8 * half)) = z;
             *reinterpret_cast<u32x4*>(Mg + PLANE8 / 2 + panel_index(CH, SUB * rb + r, SUB * cb + 8 * half)) = z;
-            *reinterpret_cast<u32x4*>(Ln + (SUB * rb + r) * LD64 + SUB * cb + 8 * half) = z;
-            *reinterpret_cast<u32x4*>(Ln + LN_PLANE + (SUB * rb + r) * LD64 + SUB * cb + 8 * half) = z;
+            *reinterpret_cast<u32x4*>(Tz + panel_index(CH, SUB * rb + r, SUB * cb + 8 * half)) = z;
+            *reinterpret_cast<u32x4*>(Tz + PLANE8 / 2 + panel_index(CH, SUB * rb + r, SUB * cb + 8 * half)) = z;
         }
         // ---- the diagonal blocks of T = (I + L)^-1 in f32 by forward substitution: lane (a, j) solves column j of
         // block a and leaves it as fp16 pairs (scale 2), scaled by beta_j (T' = T diag(beta)) and plain.
@@ -682,8 +683,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // ---- T' = (I + L)^-1 diag(beta) without ever forming the blocks of T below the diagonal: block forward
     // substitution on R = I (64 rows, 64 columns), held transposed in LDS ([column][row]) and solved in place.
     // Wave w owns the sixteen columns of block column w; no barrier:
-    //   Z_a = -sum_{b<a} L_ab X_b,   X_a = T'_aa R_a + T_aa Z_a.
-    // Every operand is an fp16 pair with scale 2 (L: 2^14). Blocks above the diagonal come out as the zeros they are.
+    //   Z_a = -sum_{b<a} L_ab X_b,   X_a = T'_aa R_a + T_aa Z_a,   from a = w on (the blocks above are zero).
+    // Every operand is an fp16 pair with scale 2 (L: 2^14).
     {
         uint16_t* RT = reinterpret_cast<uint16_t*>(smem + I_RT);
         uint16_t* Zs = reinterpret_cast<uint16_t*>(smem + I_Z);
@@ -706,8 +707,9 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
         uint16_t* Tg = reinterpret_cast<uint16_t*>(wsc + WS_TP);
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
+            if (a < wave) continue;               // (wave is uniform: whole iterations drop out)
             const uint4 tth = frag(TT, LDT, SUB * a, 0, lane), ttl = frag(TT + TT_PLANE, LDT, SUB * a, 0, lane);
-            if (a > 0) {
+            if (a > wave) {
                 // Z tile [16 rows j][16 columns c]: a lane ends with four consecutive rows of one column
                 f32x4 z = zero;
                 z = mfma_hl(frag(Ln, LD64, SUB * a, 0, lane), frag(Ln + LN_PLANE, LD64, SUB * a, 0, lane),
@@ -726,7 +728,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             const int off_z = I_Z + ((wave * SUB + cl) * LDZ + 8 * ((lane >> 4) - 2)) * 2;
             uint4 rzh = *reinterpret_cast<const uint4*>(smem + (lane < 32 ? off_r : off_z));
             uint4 rzl = *reinterpret_cast<const uint4*>(smem + (lane < 32 ? off_r + RT_PLANE * 2 : off_z + Z_PLANE * 2));
-            if (a == 0) {                         // Z_0 = 0
+            if (a == wave) {                      // Z_w = 0
                 const uint32_t keep = lane < 32 ? 0xffffffffu : 0u;
                 rzh = make_uint4(rzh.x & keep, rzh.y & keep, rzh.z & keep, rzh.w & keep);
                 rzl = make_uint4(rzl.x & keep, rzl.y & keep, rzl.z & keep, rzl.w & keep);
