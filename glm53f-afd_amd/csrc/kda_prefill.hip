@@ -860,8 +860,10 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
         const unsigned off_k = (unsigned)(WS_KGT + ((32 * wave + cl) * 32 + 8 * (lane >> 4)) * 2);  // + 1024 mt + 8192 ks
         const unsigned off_v = (unsigned)(WS_VT + ((NV * vb + value_col(0, cl)) * CH + SUB * wave + rl) * 2);   // + 512 nt
         const unsigned off_e = (unsigned)(WS_E + (32 * wave + rl) * 4);                             // + 64 mt
-        // The loads of chunk C_ into operand set X_, one group at a time (each group is requested as soon as the
-        // chunk two before it has used those registers). Unconditional: past the end they repeat the last chunk.
+        // The loads of chunk C_ into the operand set X_, one group at a time: each group is requested again, for the
+        // next chunk, as soon as this chunk has used it, so a request has all but one phase of a chunk to arrive (a
+        // second set, requested two chunks ahead, costs 80 registers and measured 2 % slower).
+        // Unconditional: past the end they repeat the last chunk.
 #define KDA_LOAD_KD(X_, C_)                                                                                         \
         {                                                                                                           \
             const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
@@ -871,19 +873,23 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                        \
                 X_.v[nt] = *reinterpret_cast<const uint2*>(src_ + off_v + 512 * nt);                                 \
         }
-#define KDA_LOAD_KE(X_, C_)                                                                                         \
+#define KDA_LOAD_K(X_, C_)                                                                                          \
         {                                                                                                           \
             const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
-            _Pragma("unroll") for (int mt = 0; mt < 2; ++mt) {                                                      \
+            _Pragma("unroll") for (int mt = 0; mt < 2; ++mt)                                                        \
                 _Pragma("unroll") for (int pl = 0; pl < 2; ++pl)                                                    \
                     _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                \
                         X_.k[pl][mt][ks] = *reinterpret_cast<const u32x4*>(src_ + PLANE16 * pl + off_k + 1024 * mt + 8192 * ks); \
-                X_.e[mt] = *reinterpret_cast<const f32x4*>(src_ + off_e + 64 * mt);                                  \
-            }                                                                                                       \
         }
-        // Chunk c with the operands in x; each group of x is then requested again for chunk c + 2.
+#define KDA_LOAD_E(X_, C_)                                                                                          \
+        {                                                                                                           \
+            const unsigned char* src_ = wsh + (long long)(C_) * WS_BYTES;                                           \
+            _Pragma("unroll") for (int mt = 0; mt < 2; ++mt)                                                        \
+                X_.e[mt] = *reinterpret_cast<const f32x4*>(src_ + off_e + 64 * mt);                                  \
+        }
+        // Chunk c with the operands in x; each group of x is then requested again for chunk c + 1.
         auto chunk_step = [&](const int c, StateOperands& x) __attribute__((always_inline)) {
-            const int c2 = min(c + 2, nch - 1);
+            const int c2 = min(c + 1, nch - 1);
             // S^T as an fp16 pair (scale 4) for the products of the chunk
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
@@ -928,6 +934,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) accS[mt][nt][r] *= x.e[mt][r];
+            KDA_LOAD_E(x, c2)
             __syncthreads();
             // S <- e^{G_last} S + Kg^T V'
 #pragma unroll
@@ -944,7 +951,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
                     for (int nt = 0; nt < NT; ++nt)
                         accS[mt][nt] = mfma_hl(as_u4(x.k[0][mt][ks]), as_u4(x.k[1][mt][ks]), vh[nt], vl[nt], accS[mt][nt]);
             }
-            KDA_LOAD_KE(x, c2)
+            KDA_LOAD_K(x, c2)
             if constexpr (sizeof(S) == 2) {
                 // a bf16 state is rounded at the end of every chunk, so the result does not depend on where passes
                 // end (the power-of-two units do not change which bits are kept)
@@ -957,21 +964,14 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             }
         };
         if (nch > 0) {
-            StateOperands xa, xb;                 // even and odd chunks
-            KDA_LOAD_KD(xa, 0) KDA_LOAD_KE(xa, 0)
-            const int c1 = min(1, nch - 1);
-            KDA_LOAD_KD(xb, c1) KDA_LOAD_KE(xb, c1)
-            // in pairs, so that the operand sets are compile-time choices; an odd last chunk follows
-            int c = 0;
+            StateOperands x;
+            KDA_LOAD_KD(x, 0) KDA_LOAD_K(x, 0) KDA_LOAD_E(x, 0)
 #pragma unroll 1
-            for (; c + 1 < nch; c += 2) {
-                chunk_step(c, xa);
-                chunk_step(c + 1, xb);
-            }
-            if (c < nch) chunk_step(c, xa);
+            for (int c = 0; c < nch; ++c) chunk_step(c, x);
         }
 #undef KDA_LOAD_KD
-#undef KDA_LOAD_KE
+#undef KDA_LOAD_K
+#undef KDA_LOAD_E
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -1026,7 +1026,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             }
         };
         auto chunk_step = [&](const int c, ReadoutOperands& x) __attribute__((always_inline)) {
-            const int c2 = min(c + 2, nch - 1);
+            const int c2 = min(c + 1, nch - 1);
             __syncthreads();                      // the chunk's state is in LDS
             if (st_c >= 0) store_rows();
             // Y^T = S^T Qg^T + V'^T M^T, the state and V' on the row side of the tiles, so that a lane ends up with four
@@ -1074,17 +1074,10 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             st_c = c;
         };
         if (nch > 0) {
-            ReadoutOperands xa, xb;
-            KDA_LOAD_T(xa, 0) KDA_LOAD_Q(xa, 0) KDA_LOAD_M(xa, 0)
-            const int c1 = min(1, nch - 1);
-            KDA_LOAD_T(xb, c1) KDA_LOAD_Q(xb, c1) KDA_LOAD_M(xb, c1)
-            int c = 0;
+            ReadoutOperands x;
+            KDA_LOAD_T(x, 0) KDA_LOAD_Q(x, 0) KDA_LOAD_M(x, 0)
 #pragma unroll 1
-            for (; c + 1 < nch; c += 2) {
-                chunk_step(c, xa);
-                chunk_step(c + 1, xb);
-            }
-            if (c < nch) chunk_step(c, xa);
+            for (int c = 0; c < nch; ++c) chunk_step(c, x);
             store_rows();
         }
 #undef KDA_LOAD_T
