@@ -52,11 +52,14 @@ constexpr int WS_M = 98304;               // fp16 x 2 [2 column panels][64 rows]
 constexpr int WS_TP = 114688;             // fp16 x 2 [2 column panels][64 rows][32 columns]: T', scale 2
 constexpr int WS_VT = 131072;             // bf16 [128 values][64 rows]: v, exact
 constexpr int WS_E = 147456;              // f32 [128 keys]: e^{G_last}
-constexpr int WS_BYTES = 147968;
+constexpr int WS_VMAX = 147968;           // f32 [4 sub-chunks]: the largest |v| of each sub-chunk's rows (all 128 values)
+constexpr int WS_CARRY = 147984;          // int [4 value blocks], in a pass's first chunk only: the serial pass before it
+                                          //   leaves here the exponent term of the next chunk's scale (chunk_scale)
+constexpr int WS_BYTES = 148096;             // (a multiple of 128: every slot starts on a cache line)
 constexpr float SC_K = 16384.0f;          // Kd, Kg, L
 constexpr float SC_Q = 131072.0f;         // Qg, M
 constexpr float SC_T = 2.0f;              // T, T', and the solve's right-hand sides
-constexpr float SC_V = 4.0f;              // S, P, V'
+static_assert(SC_K == 16384.0f && SC_Q == 131072.0f, "inter_kernel writes these as the exponents 14 and 17");
 // Element index of (row, k) in a panelled matrix with `rows` rows.
 __device__ __forceinline__ int panel_index(int rows, int row, int k) { return ((k >> 5) * rows + row) * 32 + (k & 31); }
 // LDS row strides in 16-bit elements: 128- and 64-wide operand rows padded by 16 bytes, so that the sixteen
@@ -337,6 +340,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     // from L, T' and the state update, and their outputs are never stored.
     uint32_t qr[16], kr[16];                      // bf16 pairs: the conv outputs are bf16 values
     float ssq = 0.0f, ssk = 0.0f;
+    float vmx = 0.0f;                             // the largest |v| among this lane's values (before the bf16 rounding)
     {
         // The conv's tap 3 is the lane's own row; the three rows before it are the own rows of the lanes below, a
         // DPP shift away. Lanes 0..2 of a sub-chunk also need the three rows before the sub-chunk (the conv window,
@@ -394,6 +398,7 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 if (seg == 1) { kr[4 * p + d] = pair; ssk = dot2_bf16(pair, pair, ssk); }
                 if (seg == 2) {
                     // v, transposed into VT four rows at a time: two words are four values of the row
+                    vmx = fmaxf(vmx, fmaxf(fabsf(s2[0]), fabsf(s2[1])));
                     vb2[d & 1] = pair;
                     if (d & 1) {
                         const f32x4 x = transpose16_bf(vb2[0], vb2[1], ident_bf);
@@ -444,6 +449,18 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
     }
     if (t < CH) {
         beta_s[t] = t < n ? bfround(fast_sigmoid(bf2f(b_raw))) : 0.0f;
+    }
+    {
+        // the largest |v| of the wave's sixteen rows, for the serial pass (chunk_scale), which takes the largest of a
+        // chunk's four; the margin covers the rounding of v to bf16, which can lengthen a value by 2^-8 of itself
+        vmx = fmaxf(vmx, lane_xor16<1>(vmx));
+        vmx = fmaxf(vmx, lane_xor16<2>(vmx));
+        vmx = fmaxf(vmx, lane_xor16<4>(vmx));
+        vmx = fmaxf(vmx, lane_xor16<8>(vmx));
+        const int vi = __float_as_int(vmx);
+        vmx = fmaxf(fmaxf(__int_as_float(__builtin_amdgcn_readlane(vi, 0)), __int_as_float(__builtin_amdgcn_readlane(vi, 16))),
+                    fmaxf(__int_as_float(__builtin_amdgcn_readlane(vi, 32)), __int_as_float(__builtin_amdgcn_readlane(vi, 48))));
+        if (lane == 0) reinterpret_cast<float*>(wsc + WS_VMAX)[wave] = vmx * 1.0078125f;
     }
     __syncthreads();
     // v leaves for the workspace ([value][row], as the inter pass adds it to its accumulators): its place in LDS
@@ -760,7 +777,48 @@ constexpr int S_PLANE = NV * LD128, P_PLANE = NV * LD64;   // elements from a hi
 constexpr int N_S = 0;                            // fp16 x 2 [NV][LD128]: the state, transposed
 constexpr int N_P = N_S + 2 * S_PLANE * 2;    // fp16 x 2 [NV][LD64]: P, transposed
 constexpr int N_V = N_P + 2 * P_PLANE * 2;        // fp16 x 2 [NV][LD64]: V', transposed
-constexpr int INTER_LDS = N_V + 2 * P_PLANE * 2;
+constexpr int N_X = N_V + 2 * P_PLANE * 2;         // int [4]: per state wave, the exponent of the largest |S| entering the chunk
+constexpr int INTER_LDS = N_X + 16;
+
+// The scale of S, P and V' in a chunk. Those three pass through fp16 pairs, so they are carried times a power of two,
+// 2^es, chosen per chunk from a bound on everything the chunk can produce. With N a bound on the 2-norm of every value
+// column of the state entering the chunk and m the largest |v| in it: k is normalised, beta and the decay are at most
+// one, so every row of the recurrence lengthens a column by at most m, and an entry of S, of P = V - Kd S and of
+// V' = T' P (the recurrence's own deltas) stays below N + 64 m. N follows the state one chunk behind, which keeps the
+// bookkeeping off the chain: for chunk c + 1 it is sqrt(128) times the largest entry of the state that entered
+// chunk c (measured by the state waves while they wait for that chunk's V', read by everyone behind the chunk's
+// last matrix products) plus chunk c's 64 m. Only exponents are kept (integers: no rounding, so the scales, and
+// with them every bit of the result, do not depend on where the passes are cut): with |x| < 2^(e + 1) written
+// e(x), the terms of the bound are below 2^(e(S) + 5) and 2^(e(m) + 7), their sum below 2^(E + 2) with E the
+// largest of the exponents, and es = 15 - (E + 2) puts everything below 2^15, half of fp16's largest number; what
+// the exponents round up costs at most four of the pairs' forty bits of range below the bound. A launch's first
+// chunk takes its term from the state it loads (a request's first rows) or from what the launch before left in
+// the workspace (WS_CARRY). es is kept in [-50, 50]: a state beyond 2^61 (2e18) becomes infinite, below 2^-39 the
+// pairs' absolute floor of 2^-75 shows. What one scale per chunk cannot follow is a state that collapses by more
+// than 2^25 inside a chunk while the values stay small: the next chunk still carries the old bound, and values
+// more than 2^40 below it are lost to that chunk.
+constexpr int kScaleMin = -50, kScaleMax = 50;
+__device__ __forceinline__ int exponent_of(uint32_t bits) { return (int)((bits >> 23) & 0xffu) - 127; }   // |x| < 2^(e + 1)
+// es from X (the largest exponent term of the chunks before) and the exponent of this chunk's largest |v|
+__device__ __forceinline__ int chunk_scale(int x, int ev) { return min(max(15 - (max(x, ev + 7) + 2), kScaleMin), kScaleMax); }
+__device__ __forceinline__ float pow2i(int e) { return __uint_as_float((uint32_t)(e + 127) << 23); }   // -126 <= e <= 127
+// The largest |x| over a wave's accumulators as a bit pattern, the same in every lane (the patterns of non-negative
+// floats order like unsigned integers: integer maxima, no conversions).
+__device__ __forceinline__ uint32_t wave_max_abs_bits(const f32x4 (&a)[2][NT]) {
+    uint32_t m = 0u;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) m = max(m, __float_as_uint(a[mt][nt][r]) & 0x7fffffffu);
+    m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xf, 0xf, true));       // lanes ^ 1
+    m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xf, 0xf, true));       // lanes ^ 2
+    m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x124, 0xf, 0xf, true));      // rotate by 4 inside a row of 16
+    m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x128, 0xf, 0xf, true));      // rotate by 8
+    return max(max((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
+               max((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
+}
 
 template <typename S>
 __device__ __forceinline__ float load_state_elem4(const S* p, float (&v)[4]);
@@ -809,9 +867,9 @@ __device__ __forceinline__ int value_col(int nt, int m) { return 8 * (m >> 2) + 
 
 // Pass 2: one head's NV value columns of one request through the chunks of the pass, in order. The state
 // S[128 keys][NV] lives in the MFMA accumulators of the state waves (wave w owns keys 32 w .. 32 w + 31), in units of
-// 2^16 S, the product of the scales of Kg and V'. Per chunk, three barriers:
-//   state waves:    S -> LDS | P = V - Kd S -> LDS         | S <- e^{G_last} S  | S += Kg^T V'
-//   read-out waves:          | store rows c - 1; Y = Qg S  | V' = T' P -> LDS   | Y += M V'
+// 2^14 2^e S: the scale of Kg times the chunk's scale of V' (chunk_scale). Per chunk, three barriers:
+//   state waves:    S -> LDS | P = V - Kd S -> LDS         | max |S|; S <- e^{G_last} S      | S += Kg^T V'; next scale
+//   read-out waves:          | store rows c - 1; Y = Qg S  | V' = T' P -> LDS                | Y += M V'
 // so the chain from one chunk's state to the next is three products, and in every interval the read-out waves have
 // no more to do than the state waves (with the whole of Y after the third barrier they held up the next chunk's
 // first barrier: 3.4 us per chunk instead of 3.1 with the workspace in HBM, 2.6 with it in the cache behind the L2).
@@ -819,7 +877,7 @@ template <typename S>
 __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) inter_kernel(
         int H, const int32_t* __restrict__ cu_rows, int rows1, int sub0, int chunks,
         const S* state_in, S* state_out, const long long* __restrict__ state_off,
-        bf16_t* __restrict__ out, long long out_stride, const unsigned char* __restrict__ ws) {
+        bf16_t* __restrict__ out, long long out_stride, const unsigned char* __restrict__ ws, unsigned char* carry_ws) {
     extern __shared__ __align__(16) unsigned char smem[];
     // Workgroups go to the eight XCDs round robin by their linear index. The value-column blocks of one head
     // read the same Kd, Qg, Kg, M and T', so they are spaced H apart (a multiple of 8 for the model's 64 heads):
@@ -840,14 +898,56 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
     uint16_t* Pl = reinterpret_cast<uint16_t*>(smem + N_P);
     uint16_t* Vl = reinterpret_cast<uint16_t*>(smem + N_V);
     const unsigned char* wsh = ws + ((long long)b * H + h) * chunks * (long long)WS_BYTES;
+    // (the same slot through the pointer that may write: the carry words are only ever touched through this one)
+    int* carry = reinterpret_cast<int*>(carry_ws + ((long long)b * H + h) * chunks * (long long)WS_BYTES + WS_CARRY + 4 * vb);
     // Per-lane byte offsets of the fragments inside a chunk's workspace.
     const unsigned off_a = (unsigned)(((SUB * wave + cl) * 32 + 8 * (lane >> 4)) * 2);   // Kd, Qg, M, T': + 4096 ks
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
     auto as_u4 = [](const u32x4 v) { return make_uint4(v[0], v[1], v[2], v[3]); };
-    constexpr float S_UNITS = SC_K * SC_V;                        // the accumulators hold S_UNITS S
+    // The chunks' scales (chunk_scale), the same integers in every wave of the workgroup. ev_*: the exponents of the
+    // largest |v| of the chunk before, this chunk and the next. The one after the next is requested at the top of
+    // a chunk's iteration and turned into an exponent at its end (the conversion waits for the load; loaded words
+    // that live across the loop's back edge cost a register copy there, with a wait for the load in front of it).
+    auto ev_request = [&](int c) {
+        return *reinterpret_cast<const u32x4*>(wsh + (long long)min(c, nch - 1) * WS_BYTES + WS_VMAX);
+    };
+    auto ev_of = [](const u32x4 v) {                               // (positive floats order like their bit patterns)
+        return __builtin_amdgcn_readfirstlane(exponent_of(max(max(v[0], v[1]), max(v[2], v[3]))));
+    };
+    int* mx = reinterpret_cast<int*>(smem + N_X);
+    // The exponent of the largest |S| that entered the chunk, over the four state waves.
+    auto state_exponent = [&]() {
+        const u32x4 m4 = *reinterpret_cast<const u32x4*>(mx);
+        return __builtin_amdgcn_readfirstlane(max(max((int)m4[0], (int)m4[1]), max((int)m4[2], (int)m4[3])));
+    };
+    int ev_cur = 0, ev_next = 0;
+    int x_cur = 0;                                // the next chunk's exponent term of what came before it
+    int es = 0;
+    // Chunk c's step of the bookkeeping, anywhere between its third barrier and the next chunk's first: the next
+    // chunk's scale from the state that entered chunk c and the values of chunks c and c + 1.
+    auto step = [&](const u32x4 ev_after_raw) __attribute__((always_inline)) {
+        x_cur = max(state_exponent() + 5, ev_cur + 7);
+        ev_cur = ev_next;
+        ev_next = ev_of(ev_after_raw);
+        return chunk_scale(x_cur, ev_cur);
+    };
+    // Before the first chunk: the term comes from the loaded state (whose exponent the state waves have put in mx,
+    // a barrier ago) or from the launch before.
+    // (What it loads is requested here, ahead of the state and of the first chunk's operands: vector loads arrive in
+    // order, and the first chunk's scale is needed before any of those.)
+    const int nch1 = max(nch, 1);
+    const u32x4 ev0_raw = *reinterpret_cast<const u32x4*>(wsh + WS_VMAX);
+    const u32x4 ev1_raw = *reinterpret_cast<const u32x4*>(wsh + (long long)min(1, nch1 - 1) * WS_BYTES + WS_VMAX);
+    const int carry_raw = *carry;
+    auto first_scale = [&]() __attribute__((always_inline)) {
+        ev_cur = ev_of(ev0_raw);
+        ev_next = ev_of(ev1_raw);
+        x_cur = sub0 == 0 ? state_exponent() + 5 : __builtin_amdgcn_readfirstlane(carry_raw);
+        return chunk_scale(x_cur, ev_cur);
+    };
 
     if (state_wave) {
-        // the state: accS[mt][nt][r] = S_UNITS S[key 32 w + 16 mt + rl + r][value NV vb + value_col(nt, cl)]
+        // the state: accS[mt][nt][r] = 2^eu S[key 32 w + 16 mt + rl + r][value NV vb + value_col(nt, cl)]
         f32x4 accS[2][NT];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -855,8 +955,9 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             for (int nt = 0; nt < NT; ++nt) {
                 float v4[4];
                 load_state_elem4<S>(state_in + sbase + (long long)(NV * vb + value_col(nt, cl)) * DK + 32 * wave + SUB * mt + rl, v4);
-                accS[mt][nt] = f32x4{v4[0] * S_UNITS, v4[1] * S_UNITS, v4[2] * S_UNITS, v4[3] * S_UNITS};
+                accS[mt][nt] = f32x4{v4[0], v4[1], v4[2], v4[3]};
             }
+        int eu = 0;                               // the accumulators hold 2^eu S
         const unsigned off_k = (unsigned)(WS_KGT + ((32 * wave + cl) * 32 + 8 * (lane >> 4)) * 2);  // + 1024 mt + 8192 ks
         const unsigned off_v = (unsigned)(WS_VT + ((NV * vb + value_col(0, cl)) * CH + SUB * wave + rl) * 2);   // + 512 nt
         const unsigned off_e = (unsigned)(WS_E + (32 * wave + rl) * 4);                             // + 64 mt
@@ -887,97 +988,125 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
             _Pragma("unroll") for (int mt = 0; mt < 2; ++mt)                                                        \
                 X_.e[mt] = *reinterpret_cast<const f32x4*>(src_ + off_e + 64 * mt);                                  \
         }
-        // Chunk c with the operands in x; each group of x is then requested again for chunk c + 1.
-        auto chunk_step = [&](const int c, StateOperands& x) __attribute__((always_inline)) {
-            const int c2 = min(c + 1, nch - 1);
-            // S^T as an fp16 pair (scale 4) for the products of the chunk
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    uint2 hi, lo;
-                    split_h4(scaled(accS[mt][nt], SC_V / S_UNITS), hi, lo);
-                    uint16_t* dst = Sl + (SUB * nt + cl) * LD128 + 32 * wave + SUB * mt + rl;
-                    *reinterpret_cast<uint2*>(dst) = hi;
-                    *reinterpret_cast<uint2*>(dst + S_PLANE) = lo;
-                }
-            __syncthreads();
-            // P = V - Kd S: wave w takes rows 16 w .. 16 w + 15. The workspace holds -Kd (scale 2^14), so the
-            // accumulators start at 2^16 V and end at 2^16 P.
-            f32x4 accP[NT];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const uint2 u = x.v[nt];
-                accP[nt] = f32x4{__uint_as_float(u.x << 16) * (SC_K * SC_V), __uint_as_float(u.x & 0xffff0000u) * (SC_K * SC_V),
-                                 __uint_as_float(u.y << 16) * (SC_K * SC_V), __uint_as_float(u.y & 0xffff0000u) * (SC_K * SC_V)};
-            }
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    accP[nt] = mfma_hl(as_u4(x.kd[0][ks]), as_u4(x.kd[1][ks]), frag(Sl, LD128, SUB * nt, 32 * ks, lane),
-                                       frag(Sl + S_PLANE, LD128, SUB * nt, 32 * ks, lane), accP[nt]);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                uint2 hi, lo;
-                split_h4(scaled(accP[nt], 1.0f / SC_K), hi, lo);
-                uint16_t* dst = Pl + (SUB * nt + cl) * LD64 + SUB * wave + rl;
-                *reinterpret_cast<uint2*>(dst) = hi;
-                *reinterpret_cast<uint2*>(dst + P_PLANE) = lo;
-            }
-            KDA_LOAD_KD(x, c2)
-            __syncthreads();
-            // while the read-out waves form V': the state's decay
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) accS[mt][nt][r] *= x.e[mt][r];
-            KDA_LOAD_E(x, c2)
-            __syncthreads();
-            // S <- e^{G_last} S + Kg^T V'
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                uint4 vh[NT], vl[NT];
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    vh[nt] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
-                    vl[nt] = frag(Vl + P_PLANE, LD64, SUB * nt, 32 * ks, lane);
-                }
-#pragma unroll
-                for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
-                        accS[mt][nt] = mfma_hl(as_u4(x.k[0][mt][ks]), as_u4(x.k[1][mt][ks]), vh[nt], vl[nt], accS[mt][nt]);
-            }
-            KDA_LOAD_K(x, c2)
-            if constexpr (sizeof(S) == 2) {
-                // a bf16 state is rounded at the end of every chunk, so the result does not depend on where passes
-                // end (the power-of-two units do not change which bits are kept)
-#pragma unroll
-                for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) accS[mt][nt][r] = bfround(accS[mt][nt][r]);
-            }
-        };
         if (nch > 0) {
             StateOperands x;
             KDA_LOAD_KD(x, 0) KDA_LOAD_K(x, 0) KDA_LOAD_E(x, 0)
+            if (sub0 == 0) {                      // a request's first rows: the bound comes from the state itself
+                const int e = exponent_of(wave_max_abs_bits(accS));
+                if (lane == 0) mx[wave] = e;
+                __syncthreads();
+            }
+            es = first_scale();
 #pragma unroll 1
-            for (int c = 0; c < nch; ++c) chunk_step(c, x);
+            for (int c = 0; c < nch; ++c) {
+                const int c2 = min(c + 1, nch - 1);
+                const u32x4 ev_after_raw = ev_request(c + 2);
+                // S^T as an fp16 pair for the products of the chunk, times the chunk's scale
+                {
+                    const float f = pow2i(es - eu);
+#pragma unroll
+                    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt) {
+                            uint2 hi, lo;
+                            split_h4(scaled(accS[mt][nt], f), hi, lo);
+                            uint16_t* dst = Sl + (SUB * nt + cl) * LD128 + 32 * wave + SUB * mt + rl;
+                            *reinterpret_cast<uint2*>(dst) = hi;
+                            *reinterpret_cast<uint2*>(dst + S_PLANE) = lo;
+                        }
+                }
+                __syncthreads();
+                // P = V - Kd S: wave w takes rows 16 w .. 16 w + 15. The workspace holds -Kd (scale 2^14), so the
+                // accumulators start at 2^14 2^es V and end at 2^14 2^es P.
+                f32x4 accP[NT];
+                {
+                    const float f = SC_K * pow2i(es);
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const uint2 u = x.v[nt];
+                        accP[nt] = f32x4{__uint_as_float(u.x << 16) * f, __uint_as_float(u.x & 0xffff0000u) * f,
+                                         __uint_as_float(u.y << 16) * f, __uint_as_float(u.y & 0xffff0000u) * f};
+                    }
+                }
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+                        accP[nt] = mfma_hl(as_u4(x.kd[0][ks]), as_u4(x.kd[1][ks]), frag(Sl, LD128, SUB * nt, 32 * ks, lane),
+                                           frag(Sl + S_PLANE, LD128, SUB * nt, 32 * ks, lane), accP[nt]);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    uint2 hi, lo;
+                    split_h4(scaled(accP[nt], 1.0f / SC_K), hi, lo);
+                    uint16_t* dst = Pl + (SUB * nt + cl) * LD64 + SUB * wave + rl;
+                    *reinterpret_cast<uint2*>(dst) = hi;
+                    *reinterpret_cast<uint2*>(dst + P_PLANE) = lo;
+                }
+                KDA_LOAD_KD(x, c2)
+                __syncthreads();
+                // while the read-out waves form V': the exponent of the largest entry of the state that entered the chunk
+                // (for the next chunk's scale), and the state's decay, which also takes the accumulators to this
+                // chunk's units
+                {
+                    const int e = exponent_of(wave_max_abs_bits(accS)) - eu;
+                    if (lane == 0) mx[wave] = e;
+                }
+                {
+                    const int eu_new = 14 + es;
+                    const float f = pow2i(eu_new - eu);
+                    eu = eu_new;
+#pragma unroll
+                    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) accS[mt][nt][r] *= x.e[mt][r] * f;
+                }
+                KDA_LOAD_E(x, c2)
+                __syncthreads();
+                // S <- e^{G_last} S + Kg^T V'
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    uint4 vh[NT], vl[NT];
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        vh[nt] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
+                        vl[nt] = frag(Vl + P_PLANE, LD64, SUB * nt, 32 * ks, lane);
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+                            accS[mt][nt] = mfma_hl(as_u4(x.k[0][mt][ks]), as_u4(x.k[1][mt][ks]), vh[nt], vl[nt], accS[mt][nt]);
+                }
+                KDA_LOAD_K(x, c2)
+                es = step(ev_after_raw);
+                if constexpr (sizeof(S) == 2) {
+                    // a bf16 state is rounded at the end of every chunk, so the result does not depend on where passes
+                    // end (the power-of-two units do not change which bits are kept)
+#pragma unroll
+                    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) accS[mt][nt][r] = bfround(accS[mt][nt][r]);
+                }
+            }
+            // what the next pass starts from: the term of its first chunk's scale
+            if (wave == 0 && lane == 0) *carry = x_cur;
         }
 #undef KDA_LOAD_KD
 #undef KDA_LOAD_K
 #undef KDA_LOAD_E
+        {
+            const float f = pow2i(-eu);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
+            for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-                store_state_elem4(state_out + sbase + (long long)(NV * vb + value_col(nt, cl)) * DK + 32 * wave + SUB * mt + rl,
-                                  scaled(accS[mt][nt], 1.0f / S_UNITS));
+                for (int nt = 0; nt < NT; ++nt)
+                    store_state_elem4(state_out + sbase + (long long)(NV * vb + value_col(nt, cl)) * DK + 32 * wave + SUB * mt + rl,
+                                      scaled(accS[mt][nt], f));
+        }
     } else {
         // rows of `out` that start on 16-byte boundaries take eight values per store
         const bool wide_out = ((reinterpret_cast<size_t>(out) | (size_t)(out_stride * 2)) & 15) == 0;
@@ -1007,11 +1136,12 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
         }
         f32x4 accY[NT];
         int st_c = -1;                            // the chunk whose read-out is in accY, not yet stored
+        float st_inv = 0.0f;                      //   and what takes its accumulators back to y: 2^-17 2^-es of that chunk
         auto store_rows = [&]() __attribute__((always_inline)) {
             const int nrows = min(CH, left - st_c * CH);
             if (SUB * wave + cl < nrows) {
-                // accY[nt][r] = 2^19 y[row 16 w + cl][value NV vb + 2 rl + 4 nt + r]
-                constexpr float inv = 1.0f / (SC_Q * SC_V);
+                // accY[nt][r] = 2^17 2^es y[row 16 w + cl][value NV vb + 2 rl + 4 nt + r]
+                const float inv = st_inv;
                 bf16_t* orow = out + (rr.row0 + sub0 + st_c * CH + SUB * wave + cl) * out_stride + h * DV + NV * vb + 2 * rl;
                 const u32x4 y8 = {f2bf2(accY[0][0] * inv, accY[0][1] * inv), f2bf2(accY[0][2] * inv, accY[0][3] * inv),
                                   f2bf2(accY[1][0] * inv, accY[1][1] * inv), f2bf2(accY[1][2] * inv, accY[1][3] * inv)};
@@ -1025,59 +1155,63 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
                 }
             }
         };
-        auto chunk_step = [&](const int c, ReadoutOperands& x) __attribute__((always_inline)) {
-            const int c2 = min(c + 1, nch - 1);
-            __syncthreads();                      // the chunk's state is in LDS
-            if (st_c >= 0) store_rows();
-            // Y^T = S^T Qg^T + V'^T M^T, the state and V' on the row side of the tiles, so that a lane ends up with four
-            // consecutive values of one row. The state's part now, while the state waves form P:
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) accY[nt] = zero;
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    accY[nt] = mfma_hl(frag(Sl, LD128, SUB * nt, 32 * ks, lane), frag(Sl + S_PLANE, LD128, SUB * nt, 32 * ks, lane),
-                                       as_u4(x.q[0][ks]), as_u4(x.q[1][ks]), accY[nt]);
-            KDA_LOAD_Q(x, c2)
-            __syncthreads();                      // P is in LDS
-            // V' = T' P: wave w takes rows 16 w .. 16 w + 15 (scale 2 x 4 -> 4)
-            f32x4 accV[NT];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                accV[nt] = mfma_hl(as_u4(x.t[0][0]), as_u4(x.t[1][0]), frag(Pl, LD64, SUB * nt, 0, lane),
-                                   frag(Pl + P_PLANE, LD64, SUB * nt, 0, lane), zero);
-                if (nks == 2)
-                    accV[nt] = mfma_hl(as_u4(x.t[0][1]), as_u4(x.t[1][1]), frag(Pl, LD64, SUB * nt, 32, lane),
-                                       frag(Pl + P_PLANE, LD64, SUB * nt, 32, lane), accV[nt]);
-            }
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                uint2 hi, lo;
-                split_h4(scaled(accV[nt], 1.0f / SC_T), hi, lo);
-                uint16_t* dst = Vl + (SUB * nt + cl) * LD64 + SUB * wave + rl;
-                *reinterpret_cast<uint2*>(dst) = hi;
-                *reinterpret_cast<uint2*>(dst + P_PLANE) = lo;
-            }
-            KDA_LOAD_T(x, c2)
-            __syncthreads();                      // V' is in LDS
-            // the rest of Y, while the state waves update the state
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                accY[nt] = mfma_hl(frag(Vl, LD64, SUB * nt, 0, lane), frag(Vl + P_PLANE, LD64, SUB * nt, 0, lane),
-                                   as_u4(x.m[0][0]), as_u4(x.m[1][0]), accY[nt]);
-                if (nks == 2)
-                    accY[nt] = mfma_hl(frag(Vl, LD64, SUB * nt, 32, lane), frag(Vl + P_PLANE, LD64, SUB * nt, 32, lane),
-                                       as_u4(x.m[0][1]), as_u4(x.m[1][1]), accY[nt]);
-            }
-            KDA_LOAD_M(x, c2)
-            st_c = c;
-        };
         if (nch > 0) {
             ReadoutOperands x;
             KDA_LOAD_T(x, 0) KDA_LOAD_Q(x, 0) KDA_LOAD_M(x, 0)
+            if (sub0 == 0) __syncthreads();
+            es = first_scale();
 #pragma unroll 1
-            for (int c = 0; c < nch; ++c) chunk_step(c, x);
+            for (int c = 0; c < nch; ++c) {
+                const int c2 = min(c + 1, nch - 1);
+                const u32x4 ev_after_raw = ev_request(c + 2);
+                __syncthreads();                      // the chunk's state is in LDS
+                if (st_c >= 0) store_rows();
+                // Y^T = S^T Qg^T + V'^T M^T, the state and V' on the row side of the tiles, so that a lane ends up with four
+                // consecutive values of one row. The state's part now, while the state waves form P:
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) accY[nt] = zero;
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+                        accY[nt] = mfma_hl(frag(Sl, LD128, SUB * nt, 32 * ks, lane), frag(Sl + S_PLANE, LD128, SUB * nt, 32 * ks, lane),
+                                           as_u4(x.q[0][ks]), as_u4(x.q[1][ks]), accY[nt]);
+                KDA_LOAD_Q(x, c2)
+                __syncthreads();                      // P is in LDS
+                // V' = T' P: wave w takes rows 16 w .. 16 w + 15 (the scale of T' taken out again)
+                f32x4 accV[NT];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    accV[nt] = mfma_hl(as_u4(x.t[0][0]), as_u4(x.t[1][0]), frag(Pl, LD64, SUB * nt, 0, lane),
+                                       frag(Pl + P_PLANE, LD64, SUB * nt, 0, lane), zero);
+                    if (nks == 2)
+                        accV[nt] = mfma_hl(as_u4(x.t[0][1]), as_u4(x.t[1][1]), frag(Pl, LD64, SUB * nt, 32, lane),
+                                           frag(Pl + P_PLANE, LD64, SUB * nt, 32, lane), accV[nt]);
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    uint2 hi, lo;
+                    split_h4(scaled(accV[nt], 1.0f / SC_T), hi, lo);
+                    uint16_t* dst = Vl + (SUB * nt + cl) * LD64 + SUB * wave + rl;
+                    *reinterpret_cast<uint2*>(dst) = hi;
+                    *reinterpret_cast<uint2*>(dst + P_PLANE) = lo;
+                }
+                KDA_LOAD_T(x, c2)
+                __syncthreads();                      // V' is in LDS
+                // the rest of Y, while the state waves update the state
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    accY[nt] = mfma_hl(frag(Vl, LD64, SUB * nt, 0, lane), frag(Vl + P_PLANE, LD64, SUB * nt, 0, lane),
+                                       as_u4(x.m[0][0]), as_u4(x.m[1][0]), accY[nt]);
+                    if (nks == 2)
+                        accY[nt] = mfma_hl(frag(Vl, LD64, SUB * nt, 32, lane), frag(Vl + P_PLANE, LD64, SUB * nt, 32, lane),
+                                           as_u4(x.m[0][1]), as_u4(x.m[1][1]), accY[nt]);
+                }
+                st_inv = pow2i(-17 - es);
+                es = step(ev_after_raw);
+                KDA_LOAD_M(x, c2)
+                st_c = c;
+            }
             store_rows();
         }
 #undef KDA_LOAD_T
@@ -1276,7 +1410,7 @@ int launch(int32_t heads, int32_t batch, const int32_t* cu_rows, int32_t rows1, 
         }
         const S* s_in = sub0 == 0 ? state_in : state_out;
         inter_kernel<S><<<dim3(heads * VBLOCKS, batch), INTER_THREADS, INTER_LDS, st>>>(
-            heads, cu_rows, rows1, (int)sub0, (int)chunks, s_in, state_out, soff, bfp(out), out_stride, ws);
+            heads, cu_rows, rows1, (int)sub0, (int)chunks, s_in, state_out, soff, bfp(out), out_stride, ws, ws);
         const int rc = (int)hipGetLastError();
         if (rc != 0) return rc;
         if (max_rows == 0) break;

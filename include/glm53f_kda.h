@@ -170,8 +170,8 @@ int glm53f_kda_conv_shift_batch(int32_t channels, int32_t layers, int32_t batch,
 
 /**
  * Bytes of workspace for the prefill to run `rows_per_pass` rows of every request per pass; 0 on bad
- * arguments. On this build a chunk is 64 rows and costs 147,968 bytes per head and request (every operand of the
- * state-carrying pass as a pair of fp16 planes). Replaces glm53f_kda_prefill_workspace_bytes (header :204,
+ * arguments. On this build a chunk is 64 rows and costs 148,096 bytes per head and request (every operand of the
+ * state-carrying pass as a pair of fp16 planes, and 128 bytes of per-chunk scale bookkeeping). Replaces glm53f_kda_prefill_workspace_bytes (header :204,
  * kda_prefill.cu:695-698; 34,816 bytes per 16 rows there).
  */
 int64_t glm53f_kda_prefill_workspace_bytes(int32_t heads, int32_t batch, int32_t rows_per_pass);
@@ -189,10 +189,15 @@ int64_t glm53f_kda_prefill_workspace_bytes(int32_t heads, int32_t batch, int32_t
  * Against the chain: f32 states agree to about 1e-6 normwise (1e-4 where decay is slow enough that thousands of
  * rows are remembered) and about 0.05 % of the bf16 outputs fall on the other side of a rounding boundary; not bit
  * for bit. Results do not depend on the workspace size or on how requests are batched.
- * Domain: the state, V - Kd S and V' pass through fp16 with scale 4, so the 2-norm of a value row of the state
- * (its 128 keys) plus |v| must stay below 16,376 - states below 1,400 in magnitude always do - and those three carry
- * an absolute error floor of 7.5e-9. Beyond that the state comes out non-finite where the f32 recurrence (and
- * glm53f_kda_chain) stays finite. The device arrays are not inspected on the host.
+ * Domain: the state, V - Kd S and V' pass through fp16 pairs times a power of two that the state-carrying pass
+ * chooses per chunk from a bound on everything the chunk can produce (the largest entry of the state that entered
+ * the chunk before, and the largest |v| of both chunks), so states from 2^-39 to 2^61 in magnitude come out with the
+ * same relative accuracy and a finite state stays finite, as in the f32 recurrence and in glm53f_kda_chain. One scale
+ * per chunk spans 2^40 below the chunk's bound: when a state collapses by more than 2^25 inside one chunk (every
+ * channel decaying by half every few rows, from a state that large against its values), the read-outs of the rows
+ * that lie further below the bound than that lose their accuracy, and so do, for the one chunk that follows, values
+ * more than 2^40 below the old bound. A non-finite state stays non-finite. The device arrays are not inspected on
+ * the host.
  * The first call on a device also sets two kernel attributes (LDS above 64 KiB) under a lock; make one call on
  * each device before capturing a stream. Replaces glm53f_kda_prefill (header :223-232, kda_prefill.cu:700-710).
  */

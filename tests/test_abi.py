@@ -40,6 +40,6 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_workspace_bytes_is_a_pure_host_function():
-    assert ffi.glm53f_kda_prefill_workspace_bytes(64, 1, 2048) == 32 * 147968 * 64
-    assert ffi.glm53f_kda_prefill_workspace_bytes(64, 1, 1) == 147968 * 64
+    assert ffi.glm53f_kda_prefill_workspace_bytes(64, 1, 2048) == 32 * 148096 * 64
+    assert ffi.glm53f_kda_prefill_workspace_bytes(64, 1, 1) == 148096 * 64
     assert ffi.glm53f_kda_prefill_workspace_bytes(0, 1, 16) == 0
