@@ -139,11 +139,11 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
         __syncthreads();
         if (!live) continue;
         while (k0 < pw) {                         // in pairs, so that the two register sets are compile-time choices
-            if (M <= 4 || k0 + STEP * UNROLL < pw) request(wb, k0 + STEP * UNROLL);   // (short pieces: no loads past the end)
+            request(wb, k0 + STEP * UNROLL);        // (unconditional: past the piece's end a request repeats its last step)
             work(wa, k0);
             k0 += STEP * UNROLL;
             if (k0 >= pw) break;
-            if (M <= 4 || k0 + STEP * UNROLL < pw) request(wa, k0 + STEP * UNROLL);
+            request(wa, k0 + STEP * UNROLL);
             work(wb, k0);
             k0 += STEP * UNROLL;
         }
@@ -460,9 +460,9 @@ int32_t launch_mo(const uint16_t* x, long long ldx, long long x_gs, const uint16
                   long long o_gs, hipStream_t stream) {
     const int kc = k / ksplit;
     // the widest piece of the K range whose activations fit 32 KiB (64 KiB for one row: no second piece up to
-    // k = 16,384; and from five rows up, where a 32 KiB piece would be shorter than the steps requested together
-    // and every piece's first loads wait behind a barrier: o_proj with eight rows 34.7 -> 31.6 us), a multiple of 256
-    int kp = (M == 1 || M > 4 ? LDS_BYTES : LDS_BYTES / 2) / (4 * M) / STEP * STEP;
+    // k = 16,384), a multiple of 256. (This kernel serves one to four rows: launch_m.)
+    static_assert(M <= 4, "five rows and more take gemv_wide_kernel or gemv_split_rows_kernel");
+    int kp = (M == 1 ? LDS_BYTES : LDS_BYTES / 2) / (4 * M) / STEP * STEP;
     if (kp > kc) kp = kc;
     const size_t lds = (size_t)M * kp * 4;
     const int block_outs = (THREADS / 32) * OUTS;
@@ -571,19 +571,31 @@ extern "C" int32_t glm53f_fwd_gemv_ksplit(int32_t groups, int32_t n, int32_t k) 
     return best;
 }
 
-// The reference's checks in the reference's order (gemv_bf16.cu:158-164).
+namespace fwd_gemv {
+namespace {
+// The reference's checks in the reference's order (gemv_bf16.cu:158-164); `scratch_given` stands for the two
+// scratch pointers of a split call.
+bool arguments_ok(const uint16_t* x, int64_t ldx, int64_t x_gstride, const uint16_t* w, int64_t ldw, int64_t w_gstride,
+                  int32_t groups, int32_t rows, int32_t n, int32_t k, int32_t ksplit, bool scratch_given, const void* out,
+                  int64_t ldo) {
+    if (groups < 1 || groups > 65535 || rows < 1 || rows > 8 || n < 8 || n % 8 || k < 8 || k % 8 || ksplit < 1 ||
+        ksplit > 65535 || k % ksplit || (k / ksplit) % 8)
+        return false;
+    if (!x || !w || !aligned16(x) || !aligned16(w) || !out || ldx % 8 || ldw % 8 || x_gstride % 8 || w_gstride % 8 ||
+        ldx < k || ldw < k || ldo < n)
+        return false;
+    return ksplit == 1 || scratch_given;
+}
+}  // namespace
+}  // namespace fwd_gemv
+
 extern "C" int32_t glm53f_fwd_gemv_bf16(const uint16_t* x, int64_t ldx, int64_t x_gstride, const uint16_t* w,
                                         int64_t ldw, int64_t w_gstride, int32_t groups, int32_t rows, int32_t n,
                                         int32_t k, int32_t ksplit, float* partials, uint32_t* sync, void* out,
                                         int32_t out_f32, int64_t ldo, int64_t o_gstride, ihipStream_t* stream) {
     using namespace fwd_gemv;
-    if (groups < 1 || groups > 65535 || rows < 1 || rows > 8 || n < 8 || n % 8 || k < 8 || k % 8 || ksplit < 1 ||
-        ksplit > 65535 || k % ksplit || (k / ksplit) % 8)
+    if (!arguments_ok(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, partials && sync, out, ldo))
         return kInvalid;
-    if (!x || !w || !aligned16(x) || !aligned16(w) || !out || ldx % 8 || ldw % 8 || x_gstride % 8 || w_gstride % 8 ||
-        ldx < k || ldw < k || ldo < n)
-        return kInvalid;
-    if (ksplit > 1 && (!partials || !sync)) return kInvalid;
     return out_f32 ? launch<true>(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, partials, sync, out,
                                   ldo, o_gstride, stream)
                    : launch<false>(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, partials, sync,
@@ -591,12 +603,14 @@ extern "C" int32_t glm53f_fwd_gemv_bf16(const uint16_t* x, int64_t ldx, int64_t 
 }
 
 // The same GEMV with the split-K scratch in the library's own per-GPU array: no allocation anywhere on the path.
+// Every argument is checked before anything is enqueued: a rejected call leaves the stream (and a graph under
+// capture) and the shared array untouched.
 extern "C" int32_t glm53f_fwd_gemv_bf16_static(const uint16_t* x, int64_t ldx, int64_t x_gstride, const uint16_t* w,
                                                int64_t ldw, int64_t w_gstride, int32_t groups, int32_t rows, int32_t n,
                                                int32_t k, int32_t ksplit, void* out, int32_t out_f32, int64_t ldo,
                                                int64_t o_gstride, ihipStream_t* stream) {
     using namespace fwd_gemv;
-    if (groups < 1 || rows < 1 || rows > 8 || n < 8 || ksplit < 1) return kInvalid;
+    if (!arguments_ok(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, true, out, ldo)) return kInvalid;
     float* partials = nullptr;
     unsigned* counters = nullptr;
     if (ksplit > 1) {
@@ -609,10 +623,14 @@ extern "C" int32_t glm53f_fwd_gemv_bf16_static(const uint16_t* x, int64_t ldx, i
         if (rc != 0) return rc;
         partials = reinterpret_cast<float*>(base);
         counters = reinterpret_cast<unsigned*>(base + kStaticPartialFloats * 4);
+        // The counters start at zero whatever an earlier call left behind (a kernel's last workgroup resets its
+        // counter, so this only matters after a call that did not run to its end).
         clear_counters_kernel<<<(unsigned)((count + THREADS - 1) / THREADS), THREADS, 0, stream>>>(counters, (int)count);
         const int32_t lrc = (int32_t)hipGetLastError();
         if (lrc != 0) return lrc;
     }
-    return glm53f_fwd_gemv_bf16(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, partials, counters,
-                                out, out_f32, ldo, o_gstride, stream);
+    return out_f32 ? launch<true>(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, partials, counters,
+                                  out, ldo, o_gstride, stream)
+                   : launch<false>(x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, ksplit, partials, counters,
+                                   out, ldo, o_gstride, stream);
 }

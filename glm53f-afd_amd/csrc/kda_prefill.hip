@@ -743,6 +743,10 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
                 split_h4(scaled(z, 1.0f / SC_K), hi, lo);
                 *reinterpret_cast<uint2*>(Zs + (wave * SUB + cl) * LDZ + rl) = hi;
                 *reinterpret_cast<uint2*>(Zs + Z_PLANE + (wave * SUB + cl) * LDZ + rl) = lo;
+                // other lanes of the wave read the tile back below: the order of those LDS accesses is pinned (no
+                // instruction is emitted for either line; a wave's LDS accesses complete in order)
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
             }
             // [R_a | Z_a] of the column tile as an operand [16 columns][K = 32]: k < 16 is R_a (lanes 0..31), k >= 16
             // is Z_a (lanes 32..63): one read per plane at a per-lane offset, no branch
@@ -763,6 +767,8 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
             split_h4(scaled(x, 1.0f / SC_T), hi, lo);
             *reinterpret_cast<uint2*>(RT + (SUB * wave + cl) * LD64 + SUB * a + rl) = hi;
             *reinterpret_cast<uint2*>(RT + RT_PLANE + (SUB * wave + cl) * LD64 + SUB * a + rl) = lo;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");      // the next block's fragments of R^T read these
+            __builtin_amdgcn_wave_barrier();
             split_h4(scaled(xt, 1.0f / SC_T), hi, lo);
             *reinterpret_cast<uint2*>(Tg + panel_index(CH, SUB * a + cl, SUB * wave + rl)) = hi;
             *reinterpret_cast<uint2*>(Tg + PLANE8 / 2 + panel_index(CH, SUB * a + cl, SUB * wave + rl)) = lo;
