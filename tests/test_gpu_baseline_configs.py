@@ -304,7 +304,24 @@ def test_baseline_config3_full_size_values_from_a_restored_snapshot():
         assert es <= 1e-3 and float(np.median(per)) <= 1e-5, i
         assert nd <= 2e-3 * got16.size, i                      # roundings that fall the other way
         assert hs.rel_err(got16, lit.state) <= 2.0 ** -8, i    # one rounding to bf16
-        check_outputs(hs.subset_out(heads, sub, out[r0:r1]), lit.out, f"config 3, request {i}")
+        got_out = hs.subset_out(heads, sub, out[r0:r1])
+        check_outputs(got_out, lit.out, f"config 3, request {i}")
+        far = np.flatnonzero(np.abs(got_out.astype(np.float64) - lit.out.astype(np.float64)) > 2e-2)
+        if far.size:
+            # An output beyond 2e-2 is allowed above only as a two-step event of the contract's double rounding. Whose
+            # event it is: the f32 chain kernel (a different kernel, row by row, no chunking, no fp16 anywhere) over
+            # the same rows of the same heads, from the same restored snapshot. If the chain's output at that place
+            # is off the oracle's as well, the read-out sits on a rounding boundary of the contract itself.
+            ch = hs.chain_gpu(p4, hs.subset_conv(heads, sub, conv_before[s * cw:(s + 1) * cw]),
+                              hs.subset_state(heads, sub, state_before[s * n:(s + 1) * n]), rq, want_saves=False)
+            for j in far:
+                row, col = divmod(int(j), len(sub) * DV)
+                print(f"    output beyond 2e-2 at row {row}, head {sub[col // DV]}, value {col % DV}: oracle "
+                      f"{lit.out.reshape(-1)[j]:.6f} (read-out {lit.y.reshape(-1)[j]:.6f}), prefill {got_out.reshape(-1)[j]:.6f}, "
+                      f"chain kernel {ch.out.reshape(-1)[j]:.6f}; the chain kernel differs from the oracle in "
+                      f"{int((hs.bf16_steps(ch.out, lit.out).reshape(-1, DV)[j // DV] > 0).sum())} of that row-head's 128 outputs, "
+                      f"the prefill in {int((hs.bf16_steps(got_out, lit.out).reshape(-1, DV)[j // DV] > 0).sum())}")
+                assert hs.bf16_steps(ch.out, lit.out).reshape(-1)[j] >= 1, "the chain kernel agrees with the oracle there: the event is the prefill's own"
         # the window a request leaves is its last three q | k | v rows
         assert torch.equal(conv16[s * cw:(s + 1) * cw].view(WINDOW, c), P[r1 - 3:r1, :c]), i
     # the slot no request lives in is untouched

@@ -179,7 +179,11 @@ def test_random_ragged_batches_against_the_oracle(seed):
         # normwise 2^-7: two bf16 steps of the largest output (the read-out and the gated norm each round to bf16)
         got_rows, ref_rows = out[r0 * n:(r0 + rq.rows) * n], lit.out
         assert hs.rel_err(got_rows, ref_rows) <= OUT_REL, (label, i)
-        assert bf16_state or flips_ok(hs.ulps(got_rows, ref_rows)[1], got_rows.size), (label, i)
+        # outputs that differ at all: 0.3 % with an f32 state; with a bf16 state the state's rounding after every
+        # chunk (against the unrounded oracle) moves read-outs across boundaries too: 3 % as in the reduced
+        # configuration 3, where 1.2 % were measured
+        differ = hs.ulps(got_rows, ref_rows)[1]
+        assert differ <= max(4, (0.03 if bf16_state else FLIP_FRACTION) * got_rows.size), (label, i, differ, got_rows.size)
     for slot in set(range(slots_n)) - set(slots):
         at = pool.conv_off(slot)
         assert np.array_equal(hs.back(pool.conv[at:at + cw]), pool.conv_of(slot)), (label, slot)
