@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the KDA hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|mark|gemv|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decode|prefill|verify|mark|gemv|layer|copy]
 
 Prints ONE JSON line. The headline `value` is the decode step's state traffic in GB/s in the 16-slot decode configuration
 (16 slots x 1 token out of a 48-slot bf16 pool, 64 heads, 34 layers each with its own pool so the working set
@@ -561,6 +561,118 @@ def bench_gemv(steps, warmup, stream, cpu=True):
     return res
 
 
+
+# ------------------------------------------------------------------------------------------------ decode layer
+
+def bench_layer_decode(steps, warmup, stream):
+    """A KDA layer's decode step end to end as the engine issues it (crates/glm53f-forward/src/forward.rs:3494-3542
+    the projections, :3672-3705 the core's arguments, :3772-3789 the output projection), over all 34 layers with
+    their own weights, states and conv windows (12.8 GB: nothing is found in a cache): per layer
+        p   = normed x qkvb^T   [rows][24,640]   (q | k | v | beta logits; b_off = 24,576)
+        fga = normed x fga^T    [rows][256]      (the gates' low-rank halves; split K, so it needs scratch)
+        ag  = fga x fgb^T       [rows][2 x 8192] (two groups: forget-gate input | output-gate logits, interleaved rows)
+        core: chain + conv window advance in one launch on the slots' states (glm53f_kda_chain_shift_batch_bf16state)
+        out = kda_out x o^T     [rows][4096]
+    Up to 8 rows the projections are this library's GEMV (the split one through glm53f_fwd_gemv_bf16_static, which
+    holds its scratch itself), above that the vendor GEMM, as the reference's dispatch has it (gemm.rs:228-234);
+    benchmark configuration 1's 16 slots therefore take the vendor GEMM, and 8 slots are measured beside them for
+    the GEMV path. Each both ways: launched eagerly, and as one captured graph replayed."""
+    from glm53f_forward import ffi as fwd
+    heads, layers, slots_n, hidden = HEADS, LAYERS, 48, 4096
+    width, dim = heads * DK, DK                            # 8192, 128
+    pcols = 3 * width + heads                              # 24,640
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    n, cw = state_len(heads), WINDOW * channels(heads)
+
+    def weight(*shape):
+        w = torch.empty(*shape, dtype=torch.bfloat16, device=DEV)
+        flat = w.view(-1)
+        for i in range(0, flat.numel(), 1 << 26):           # in slices: the f32 temporaries stay small
+            j = min(flat.numel(), i + (1 << 26))
+            flat[i:j] = (torch.randn(j - i, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
+        return w
+
+    w_qkvb, w_fga = weight(layers, pcols, hidden), weight(layers, 2 * dim, hidden)
+    w_fgb, w_o = weight(layers, 2, width, dim), weight(layers, hidden, width)
+    layer = Layer(heads, gen)
+    pools = (torch.randn(layers, slots_n * n, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
+    convs = torch.randn(layers, slots_n * cw, device=DEV, generator=gen).to(torch.bfloat16)
+    weight_bytes = (pcols * hidden + 2 * dim * hidden + 2 * width * dim + hidden * width) * 2
+    # on a stream of its own (default priority): the legacy default stream cannot be captured
+    stream = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    st = stream.cuda_stream
+    res = {"config": {"workload": "a KDA layer's decode step end to end, 34 layers in turn: kda_proj, the two gate "
+                                  "projections, chain + conv window advance, o_proj; engine strides",
+                      "weight_bytes_per_layer": weight_bytes}}
+    for batch in (16, 8):
+        normed = torch.randn(batch, hidden, device=DEV, generator=gen).to(torch.bfloat16)
+        pbuf = torch.zeros(batch, pcols, dtype=torch.bfloat16, device=DEV)
+        fga = torch.zeros(batch, 2 * dim, dtype=torch.bfloat16, device=DEV)
+        ag = torch.zeros(batch, 2 * width, dtype=torch.bfloat16, device=DEV)
+        kda_out = torch.zeros(batch, width, dtype=torch.bfloat16, device=DEV)
+        attn_out = torch.zeros(batch, hidden, dtype=torch.bfloat16, device=DEV)
+        perm = torch.randperm(slots_n, generator=torch.Generator().manual_seed(12))[:batch]
+        cu = torch.arange(batch + 1, dtype=torch.int32, device=DEV)
+        soff, coff = (perm.to(torch.int64) * n).to(DEV), (perm.to(torch.int64) * cw).to(DEV)
+        core = ffi.glm53f_kda_chain_shift_batch_bf16state
+        core_args = [(heads, batch, ptr(cu), ptr(pbuf), pcols, 3 * width, ptr(ag), 2 * width, ptr(ag, width), 2 * width,
+                      ptr(convs[l]), ptr(coff), ptr(layer.conv_w), ptr(pools[l]), ptr(pools[l]), ptr(soff),
+                      *layer.args(), ptr(kda_out), width, None, None, None, None, st) for l in range(layers)]
+        gemv = batch <= 8
+        if gemv:
+            ks = {name: fwd.glm53f_fwd_gemv_ksplit(g, nn, kk) for name, g, nn, kk in
+                  (("qkvb", 1, pcols, hidden), ("fga", 1, 2 * dim, hidden), ("fgb", 2, width, dim), ("o", 1, hidden, width))}
+            gv = fwd.glm53f_fwd_gemv_bf16_static
+            gemv_args = [[
+                (ptr(normed), hidden, 0, ptr(w_qkvb[l]), hidden, 0, 1, batch, pcols, hidden, ks["qkvb"], ptr(pbuf), 0, pcols, 0, st),
+                (ptr(normed), hidden, 0, ptr(w_fga[l]), hidden, 0, 1, batch, 2 * dim, hidden, ks["fga"], ptr(fga), 0, 2 * dim, 0, st),
+                (ptr(fga), 2 * dim, dim, ptr(w_fgb[l]), dim, width * dim, 2, batch, width, dim, ks["fgb"], ptr(ag), 0, 2 * width, width, st),
+                (ptr(kda_out), width, 0, ptr(w_o[l]), width, 0, 1, batch, hidden, width, ks["o"], ptr(attn_out), 0, hidden, 0, st),
+            ] for l in range(layers)]
+        ag_f, ag_g = ag[:, :width], ag[:, width:]
+
+        def step():
+            for l in range(layers):
+                if gemv:
+                    a = gemv_args[l]
+                    check(gv(*a[0]), "kda_proj")
+                    check(gv(*a[1]), "fga")
+                    check(gv(*a[2]), "fgb")
+                else:
+                    torch.mm(normed, w_qkvb[l].t(), out=pbuf)
+                    torch.mm(normed, w_fga[l].t(), out=fga)
+                    torch.mm(fga[:, :dim], w_fgb[l, 0].t(), out=ag_f)
+                    torch.mm(fga[:, dim:], w_fgb[l, 1].t(), out=ag_g)
+                check(core(*core_args[l]), "chain + shift")
+                if gemv:
+                    check(gv(*gemv_args[l][3]), "o_proj")
+                else:
+                    torch.mm(kda_out, w_o[l].t(), out=attn_out)
+
+        with torch.cuda.stream(stream):
+            ms_eager = timed(step, steps, warmup, stream)
+            graph = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=stream):
+                step()
+            ms_graph = timed(graph.replay, steps, warmup, stream)
+        state_bytes = 2 * batch * n * 2
+        per_layer = weight_bytes + state_bytes
+        key = f"slots{batch}"
+        res[key] = {"projections": "this library's GEMV (glm53f_fwd_gemv_bf16_static)" if gemv else "vendor GEMM (hipBLASLt through torch.mm)",
+                    "eager_us_per_layer": ms_eager * 1e3 / layers, "graph_us_per_layer": ms_graph * 1e3 / layers,
+                    "bytes_per_layer": per_layer, "state_bytes_per_layer": state_bytes,
+                    "eager_GBps": per_layer / (ms_eager * 1e-3 / layers) / 1e9,
+                    "graph_GBps": per_layer / (ms_graph * 1e-3 / layers) / 1e9}
+        best = min(ms_eager, ms_graph)
+        res[key]["roofline"] = {"bound": "hbm", "achieved": per_layer / (best * 1e-3 / layers) / 1e9, "peak": HBM_PEAK_GBPS,
+                                "unit": "GB/s", "frac": per_layer / (best * 1e-3 / layers) / 1e9 / HBM_PEAK_GBPS,
+                                "traffic": None, "what": "weights of the four projections + state read and written, "
+                                                         "over the faster of the eager and the graph time"}
+        del graph
+    return res
+
 # ------------------------------------------------------------------------------------------------ main
 
 # ------------------------------------------------------------------------------------------------ copy
@@ -580,7 +692,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "gemv", "copy"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "gemv", "layer", "copy"], default=None)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -636,6 +748,12 @@ def main():
         if args.only == "gemv":
             line.update({"value": gv["roofline"]["achieved"], "ms_per_step": gv["kda_proj_1row"]["us"] / 1e3,
                          "roofline": gv["roofline"], "config": gv["config"]})
+    if args.only in (None, "layer"):
+        ly = bench_layer_decode(max(2, args.steps // 4), max(1, args.warmup // 2), stream)
+        line["layer_decode"] = ly
+        if args.only == "layer":
+            line.update({"value": ly["slots16"]["roofline"]["achieved"], "ms_per_step": ly["slots16"]["eager_us_per_layer"] * LAYERS / 1e3,
+                         "roofline": ly["slots16"]["roofline"], "config": ly["config"]})
     if args.only == "copy":
         cp = bench_copy(args.steps, args.warmup, stream)
         line.update({"copy": cp, "value": cp["GBps"], "ms_per_step": cp["ms"],
