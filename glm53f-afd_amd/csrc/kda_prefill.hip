@@ -779,10 +779,20 @@ __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2,
 }
 
 // LDS map of inter_kernel, bytes: only what the waves share, each as an fp16 pair of planes.
-constexpr int S_PLANE = NV * LD128, P_PLANE = NV * LD64;   // elements from a hi plane to its lo plane
-constexpr int N_S = 0;                            // fp16 x 2 [NV][LD128]: the state, transposed
-constexpr int N_P = N_S + 2 * S_PLANE * 2;    // fp16 x 2 [NV][LD64]: P, transposed
-constexpr int N_V = N_P + 2 * P_PLANE * 2;        // fp16 x 2 [NV][LD64]: V', transposed
+// Row strides and placement of what the waves exchange. A row is padded by 32 bytes and the 16-byte pieces of rows
+// 4..7 and 12..15 of every sixteen swap places in pairs: with that a fragment read (ds_read_b128: sixteen rows, four
+// pieces) runs at the full LDS rate and a tile store (ds_write_b64: sixteen rows, four elements) at the stores' best,
+// where 16 bytes of padding alone gave 0.63 and 0.93 of those rates (measured in a probe of the two access patterns
+// over strides and swizzles; this launch's first phase is bound by its 128 KB of fragment reads per chunk).
+constexpr int NLD128 = 144, NLD64 = 80;
+__device__ __forceinline__ int piece_swap(int row) { return ((row >> 2) & 1) << 3; }      // in 16-bit elements
+__device__ __forceinline__ uint4 nfrag(const uint16_t* base, int ld, int row0, int k0, int lane) {
+    return *reinterpret_cast<const uint4*>(base + (row0 + (lane & 15)) * ld + ((k0 + 8 * (lane >> 4)) ^ piece_swap(lane & 15)));
+}
+constexpr int S_PLANE = NV * NLD128, P_PLANE = NV * NLD64;   // elements from a hi plane to its lo plane
+constexpr int N_S = 0;                            // fp16 x 2 [NV][NLD128]: the state, transposed
+constexpr int N_P = N_S + 2 * S_PLANE * 2;    // fp16 x 2 [NV][NLD64]: P, transposed
+constexpr int N_V = N_P + 2 * P_PLANE * 2;        // fp16 x 2 [NV][NLD64]: V', transposed
 constexpr int N_X = N_V + 2 * P_PLANE * 2;         // int [4]: per state wave, the exponent of the largest |S| entering the chunk
 constexpr int INTER_LDS = N_X + 16;
 
@@ -1016,7 +1026,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
                         for (int nt = 0; nt < NT; ++nt) {
                             uint2 hi, lo;
                             split_h4(scaled(accS[mt][nt], f), hi, lo);
-                            uint16_t* dst = Sl + (SUB * nt + cl) * LD128 + 32 * wave + SUB * mt + rl;
+                            uint16_t* dst = Sl + (SUB * nt + cl) * NLD128 + ((32 * wave + SUB * mt + rl) ^ piece_swap(cl));
                             *reinterpret_cast<uint2*>(dst) = hi;
                             *reinterpret_cast<uint2*>(dst + S_PLANE) = lo;
                         }
@@ -1038,13 +1048,13 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
                 for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt)
-                        accP[nt] = mfma_hl(as_u4(x.kd[0][ks]), as_u4(x.kd[1][ks]), frag(Sl, LD128, SUB * nt, 32 * ks, lane),
-                                           frag(Sl + S_PLANE, LD128, SUB * nt, 32 * ks, lane), accP[nt]);
+                        accP[nt] = mfma_hl(as_u4(x.kd[0][ks]), as_u4(x.kd[1][ks]), nfrag(Sl, NLD128, SUB * nt, 32 * ks, lane),
+                                           nfrag(Sl + S_PLANE, NLD128, SUB * nt, 32 * ks, lane), accP[nt]);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     uint2 hi, lo;
                     split_h4(scaled(accP[nt], 1.0f / SC_K), hi, lo);
-                    uint16_t* dst = Pl + (SUB * nt + cl) * LD64 + SUB * wave + rl;
+                    uint16_t* dst = Pl + (SUB * nt + cl) * NLD64 + ((SUB * wave + rl) ^ piece_swap(cl));
                     *reinterpret_cast<uint2*>(dst) = hi;
                     *reinterpret_cast<uint2*>(dst + P_PLANE) = lo;
                 }
@@ -1076,8 +1086,8 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
                     uint4 vh[NT], vl[NT];
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) {
-                        vh[nt] = frag(Vl, LD64, SUB * nt, 32 * ks, lane);
-                        vl[nt] = frag(Vl + P_PLANE, LD64, SUB * nt, 32 * ks, lane);
+                        vh[nt] = nfrag(Vl, NLD64, SUB * nt, 32 * ks, lane);
+                        vl[nt] = nfrag(Vl + P_PLANE, NLD64, SUB * nt, 32 * ks, lane);
                     }
 #pragma unroll
                     for (int mt = 0; mt < 2; ++mt)
@@ -1180,7 +1190,7 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
                 for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt)
-                        accY[nt] = mfma_hl(frag(Sl, LD128, SUB * nt, 32 * ks, lane), frag(Sl + S_PLANE, LD128, SUB * nt, 32 * ks, lane),
+                        accY[nt] = mfma_hl(nfrag(Sl, NLD128, SUB * nt, 32 * ks, lane), nfrag(Sl + S_PLANE, NLD128, SUB * nt, 32 * ks, lane),
                                            as_u4(x.q[0][ks]), as_u4(x.q[1][ks]), accY[nt]);
                 KDA_LOAD_Q(x, c2)
                 __syncthreads();                      // P is in LDS
@@ -1188,17 +1198,17 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
                 f32x4 accV[NT];
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    accV[nt] = mfma_hl(as_u4(x.t[0][0]), as_u4(x.t[1][0]), frag(Pl, LD64, SUB * nt, 0, lane),
-                                       frag(Pl + P_PLANE, LD64, SUB * nt, 0, lane), zero);
+                    accV[nt] = mfma_hl(as_u4(x.t[0][0]), as_u4(x.t[1][0]), nfrag(Pl, NLD64, SUB * nt, 0, lane),
+                                       nfrag(Pl + P_PLANE, NLD64, SUB * nt, 0, lane), zero);
                     if (nks == 2)
-                        accV[nt] = mfma_hl(as_u4(x.t[0][1]), as_u4(x.t[1][1]), frag(Pl, LD64, SUB * nt, 32, lane),
-                                           frag(Pl + P_PLANE, LD64, SUB * nt, 32, lane), accV[nt]);
+                        accV[nt] = mfma_hl(as_u4(x.t[0][1]), as_u4(x.t[1][1]), nfrag(Pl, NLD64, SUB * nt, 32, lane),
+                                           nfrag(Pl + P_PLANE, NLD64, SUB * nt, 32, lane), accV[nt]);
                 }
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     uint2 hi, lo;
                     split_h4(scaled(accV[nt], 1.0f / SC_T), hi, lo);
-                    uint16_t* dst = Vl + (SUB * nt + cl) * LD64 + SUB * wave + rl;
+                    uint16_t* dst = Vl + (SUB * nt + cl) * NLD64 + ((SUB * wave + rl) ^ piece_swap(cl));
                     *reinterpret_cast<uint2*>(dst) = hi;
                     *reinterpret_cast<uint2*>(dst + P_PLANE) = lo;
                 }
@@ -1207,10 +1217,10 @@ __global__ void __launch_bounds__(INTER_THREADS) __attribute__((amdgpu_waves_per
                 // the rest of Y, while the state waves update the state
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    accY[nt] = mfma_hl(frag(Vl, LD64, SUB * nt, 0, lane), frag(Vl + P_PLANE, LD64, SUB * nt, 0, lane),
+                    accY[nt] = mfma_hl(nfrag(Vl, NLD64, SUB * nt, 0, lane), nfrag(Vl + P_PLANE, NLD64, SUB * nt, 0, lane),
                                        as_u4(x.m[0][0]), as_u4(x.m[1][0]), accY[nt]);
                     if (nks == 2)
-                        accY[nt] = mfma_hl(frag(Vl, LD64, SUB * nt, 32, lane), frag(Vl + P_PLANE, LD64, SUB * nt, 32, lane),
+                        accY[nt] = mfma_hl(nfrag(Vl, NLD64, SUB * nt, 32, lane), nfrag(Vl + P_PLANE, NLD64, SUB * nt, 32, lane),
                                            as_u4(x.m[0][1]), as_u4(x.m[1][1]), accY[nt]);
                 }
                 st_inv = pow2i(-17 - es);
