@@ -63,10 +63,14 @@ __device__ __forceinline__ void store_out(void* out, long long idx, float v) {
 
 // grid (ceil(n / (8 OUTS)), ksplit, groups). kp: the piece of a split's K range staged at a time (a multiple of
 // 256, rows * kp * 4 bytes of LDS). UNROLL: steps whose weight pieces are requested together.
+// inside > 1 (then gridDim.y is 1): the workgroup walks all `inside` splits of its outputs itself, one after the
+// other, and adds their sums in split order as the model does - no partial sums in memory, no counter, no fence.
+// The split exists to give a small n workgroups enough; with few splits the walk is shorter than the hand-over
+// through memory (4096 -> 256 with four splits: 13 us as four workgroups per block of outputs, 2 MB of weights).
 template <int M, int OUTS, bool F32>
 __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restrict__ x, long long ldx, long long x_gs,
                                                        const uint16_t* __restrict__ w, long long ldw, long long w_gs,
-                                                       int n, int kc, int kp, float* __restrict__ partials,
+                                                       int n, int kc, int kp, int inside, float* __restrict__ partials,
                                                        unsigned* __restrict__ sync, void* __restrict__ out,
                                                        long long ldo, long long o_gs) {
     constexpr int BLOCK_OUTS = (THREADS / 32) * OUTS;
@@ -74,9 +78,15 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
     extern __shared__ __align__(16) unsigned char smem[];
     float* xs = reinterpret_cast<float*>(smem);                       // [M][kp]
     const int t = threadIdx.x, hw = t >> 5, l = t & 31;
-    const int g = blockIdx.z, split = blockIdx.y, nsplit = gridDim.y;
+    const int g = blockIdx.z, nsplit = gridDim.y;
     const int o0 = blockIdx.x * BLOCK_OUTS + hw * OUTS;               // n % 8 == 0: o0 < n means o0 + OUTS <= n
     const bool live = o0 < n;
+    void* og = F32 ? static_cast<void*>(static_cast<float*>(out) + g * o_gs)
+                   : static_cast<void*>(static_cast<uint16_t*>(out) + g * o_gs);
+
+    float total[OUTS][M];                         // inside > 1: the splits' sums so far
+    for (int walk = 0; walk < inside; ++walk) {
+    const int split = inside > 1 ? walk : (int)blockIdx.y;
     const int lo = split * kc;
     const uint16_t* xg = x + g * x_gs + lo;
     const uint16_t* w0 = w + g * w_gs + (long long)(live ? o0 : 0) * ldw + lo;
@@ -128,7 +138,7 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
         u32x4 wa[UNROLL][OUTS], wb[UNROLL][OUTS];
         int k0 = 8 * l;
         request(wa, k0);
-        if (p0 > 0) __syncthreads();
+        if (p0 > 0 || walk > 0) __syncthreads();
         for (int e = t; e < M * (pw / 8); e += THREADS) {
             const int m = e / (pw / 8), c = e - m * (pw / 8);
             const u32x4 v = *reinterpret_cast<const u32x4*>(xg + m * ldx + p0 + 8 * c);
@@ -149,19 +159,21 @@ __global__ void __launch_bounds__(THREADS) gemv_kernel(const uint16_t* __restric
         }
     }
 
-    void* og = F32 ? static_cast<void*>(static_cast<float*>(out) + g * o_gs)
-                   : static_cast<void*>(static_cast<uint16_t*>(out) + g * o_gs);
     if (live) {
 #pragma unroll
         for (int r = 0; r < OUTS; ++r)
 #pragma unroll
             for (int m = 0; m < M; ++m) {
                 const float v = half_wave_sum(acc[r][m]);
-                if (l == ((r * M + m) & 31)) {
+                if (inside > 1) {                 // (every lane of the half-wave holds the same bits)
+                    total[r][m] = walk == 0 ? v : total[r][m] + v;
+                    if (walk == inside - 1 && l == ((r * M + m) & 31)) store_out<F32>(og, (long long)m * ldo + o0 + r, total[r][m]);
+                } else if (l == ((r * M + m) & 31)) {
                     if (nsplit > 1) partials[(((long long)g * nsplit + split) * M + m) * n + o0 + r] = v;
                     else store_out<F32>(og, (long long)m * ldo + o0 + r, v);
                 }
             }
+    }
     }
     if (nsplit == 1) return;
 
@@ -205,7 +217,7 @@ template <int M, bool F32>
 __global__ void __launch_bounds__(THREADS) gemv_split_rows_kernel(const uint16_t* __restrict__ x, long long ldx,
                                                                   long long x_gs, const uint16_t* __restrict__ w,
                                                                   long long ldw, long long w_gs, int n, int kc,
-                                                                  float* __restrict__ partials,
+                                                                  int inside, float* __restrict__ partials,
                                                                   unsigned* __restrict__ sync, void* __restrict__ out,
                                                                   long long ldo, long long o_gs) {
     constexpr int MR = (M + 1) / 2;                                   // rows of a lane: row0 .. row0 + MR - 1, below M
@@ -214,8 +226,14 @@ __global__ void __launch_bounds__(THREADS) gemv_split_rows_kernel(const uint16_t
     __shared__ __align__(16) float xs[M * kp];
     const int t = threadIdx.x, l = t & 31;
     const int row0 = ((t >> 5) & 1) * MR;
-    const int g = blockIdx.z, split = blockIdx.y, nsplit = gridDim.y;
+    const int g = blockIdx.z, nsplit = gridDim.y;
     const int o0 = blockIdx.x * SPLIT_BLOCK_OUTS + (t >> 6) * SPLIT_OUTS;   // n % 8 == 0: all eight exist
+    void* og = F32 ? static_cast<void*>(static_cast<float*>(out) + g * o_gs)
+                   : static_cast<void*>(static_cast<uint16_t*>(out) + g * o_gs);
+
+    float total[SPLIT_OUTS][MR];                  // inside > 1 (as in gemv_kernel): the splits' sums so far
+    for (int walk = 0; walk < inside; ++walk) {
+    const int split = inside > 1 ? walk : (int)blockIdx.y;
     const int lo = split * kc;
     const uint16_t* xg = x + g * x_gs + lo;
     const uint16_t* w0 = w + g * w_gs + (long long)o0 * ldw + lo;
@@ -285,7 +303,7 @@ __global__ void __launch_bounds__(THREADS) gemv_split_rows_kernel(const uint16_t
     request(wa, 0);
     request_x(0);
     for (int p0 = 0; p0 < kc; p0 += kp) {
-        if (p0 > 0) __syncthreads();              // every lane is past its reads of the piece before
+        if (p0 > 0 || walk > 0) __syncthreads();  // every lane is past its reads of the piece before
         stage_x();
         __syncthreads();
         request(wb, p0 + GROUP);
@@ -295,19 +313,21 @@ __global__ void __launch_bounds__(THREADS) gemv_split_rows_kernel(const uint16_t
         if (p0 + GROUP < kc) work(wb, p0 + GROUP, p0);
     }
 
-    void* og = F32 ? static_cast<void*>(static_cast<float*>(out) + g * o_gs)
-                   : static_cast<void*>(static_cast<uint16_t*>(out) + g * o_gs);
 #pragma unroll
     for (int r = 0; r < SPLIT_OUTS; ++r)
 #pragma unroll
         for (int mi = 0; mi < MR; ++mi) {
             const float v = half_wave_sum(acc[r][mi]);
             const int m = row0 + mi;
-            if (m < M && l == ((r * MR + mi) & 31)) {
+            if (inside > 1) {
+                total[r][mi] = walk == 0 ? v : total[r][mi] + v;
+                if (walk == inside - 1 && m < M && l == ((r * MR + mi) & 31)) store_out<F32>(og, (long long)m * ldo + o0 + r, total[r][mi]);
+            } else if (m < M && l == ((r * MR + mi) & 31)) {
                 if (nsplit > 1) partials[(((long long)g * nsplit + split) * M + m) * n + o0 + r] = v;
                 else store_out<F32>(og, (long long)m * ldo + o0 + r, v);
             }
         }
+    }
     if (nsplit == 1) return;
 
     int& last = *reinterpret_cast<int*>(xs);      // as above: the last workgroup of these eight outputs adds the splits
@@ -454,6 +474,18 @@ __global__ void __launch_bounds__(WIDE_THREADS) gemv_wide_kernel(const uint16_t*
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Whether a launch with `ksplit` splits and these shapes walks the splits inside its workgroups (gemv_kernel): up to
+// four splits, in the kernels that serve a small n. Such a launch touches neither the partial sums nor the counters.
+constexpr int kMaxSplitsInside = 4;
+#ifndef KDA_SPLIT_ROWS_FROM
+#define KDA_SPLIT_ROWS_FROM 3
+#endif
+inline bool splits_inside(int rows, int groups, int n, int ksplit) {
+    if (ksplit < 2 || ksplit > kMaxSplitsInside) return false;
+    const long long blocks8 = (long long)(n / 8) * ksplit * groups;
+    return !(rows >= 3 && blocks8 >= 4 * 512);    // (the wide kernel keeps its splits in the grid)
+}
+
 template <int M, int OUTS, bool F32>
 int32_t launch_mo(const uint16_t* x, long long ldx, long long x_gs, const uint16_t* w, long long ldw, long long w_gs,
                   int groups, int n, int k, int ksplit, float* partials, unsigned* sync, void* out, long long ldo,
@@ -466,9 +498,10 @@ int32_t launch_mo(const uint16_t* x, long long ldx, long long x_gs, const uint16
     if (kp > kc) kp = kc;
     const size_t lds = (size_t)M * kp * 4;
     const int block_outs = (THREADS / 32) * OUTS;
-    const dim3 grid((unsigned)((n + block_outs - 1) / block_outs), (unsigned)ksplit, (unsigned)groups);
-    gemv_kernel<M, OUTS, F32><<<grid, THREADS, lds, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, kc, kp, partials, sync,
-                                                              out, ldo, o_gs);
+    const int inside = splits_inside(M, groups, n, ksplit) ? ksplit : 1;
+    const dim3 grid((unsigned)((n + block_outs - 1) / block_outs), (unsigned)(inside > 1 ? 1 : ksplit), (unsigned)groups);
+    gemv_kernel<M, OUTS, F32><<<grid, THREADS, lds, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, kc, kp, inside, partials,
+                                                              sync, out, ldo, o_gs);
     return (int32_t)hipGetLastError();
 }
 
@@ -490,10 +523,11 @@ int32_t launch_m(const uint16_t* x, long long ldx, long long x_gs, const uint16_
                                                                                      partials, sync, out, ldo, o_gs);
         return (int32_t)hipGetLastError();
     }
-    if constexpr (M > 4) {
-        const dim3 grid((unsigned)(n / SPLIT_BLOCK_OUTS), (unsigned)ksplit, (unsigned)groups);
-        gemv_split_rows_kernel<M, F32><<<grid, THREADS, 0, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, k / ksplit, partials,
-                                                                     sync, out, ldo, o_gs);
+    if constexpr (M >= KDA_SPLIT_ROWS_FROM) {
+        const int inside = splits_inside(M, groups, n, ksplit) ? ksplit : 1;
+        const dim3 grid((unsigned)(n / SPLIT_BLOCK_OUTS), (unsigned)(inside > 1 ? 1 : ksplit), (unsigned)groups);
+        gemv_split_rows_kernel<M, F32><<<grid, THREADS, 0, stream>>>(x, ldx, x_gs, w, ldw, w_gs, n, k / ksplit, inside,
+                                                                     partials, sync, out, ldo, o_gs);
         return (int32_t)hipGetLastError();
     } else {
         if (n % 16 == 0 && blocks8 >= 2 * 1024)
@@ -614,10 +648,14 @@ extern "C" int32_t glm53f_fwd_gemv_bf16_static(const uint16_t* x, int64_t ldx, i
     float* partials = nullptr;
     unsigned* counters = nullptr;
     if (ksplit > 1) {
-        // beyond the array: rejected, never truncated
+        // beyond the array: rejected, never truncated (whether or not this shape's kernel goes through the array:
+        // the limit is the entry point's, not a kernel's)
         const unsigned long long floats = (unsigned long long)groups * (unsigned long long)ksplit * rows * n;
         const unsigned long long count = (unsigned long long)groups * (unsigned long long)(n / 8);
         if (floats > kStaticPartialFloats || count > kStaticCounters) return kInvalid;
+    }
+    if (ksplit > 1 && !splits_inside(rows, groups, n, ksplit)) {
+        const unsigned long long count = (unsigned long long)groups * (unsigned long long)(n / 8);
         unsigned char* base = nullptr;
         const int rc = scratch_of_current_device(&base);
         if (rc != 0) return rc;
