@@ -35,11 +35,11 @@ from glm53f_kda import DK, DV, HEADS, LAYERS, WINDOW, channels, ffi, state_len
 # offline; the summaries are kept in profiles/.
 TRAFFIC_BYTES = {
     "decode_chain": (36_798 + 33_024) * 1024,            # per plain chain launch, 16 slots x 1 row
-    "verify_chain": (167_884 + 1_585_673) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
+    "verify_chain": (167_883 + 1_585_706) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
     # two passes of 1024 rows (intra read + written, inter read + written) and one norm launch
-    "prefill_2048_rows": (2 * (73_999 + 141_345 + 144_086 + 20_480) + 65_755 + 32_912) * 1024,
-    "mark_state_pages": (69_933 + 70_868) * 1024,
-    "gemv_kda_proj_1row": (197_903 + 48) * 1024,         # per launch: the weights once, the activations, the outputs
+    "prefill_2048_rows": (2 * (74_012 + 141_316 + 144_138 + 20_482) + 65_755 + 32_912) * 1024,
+    "mark_state_pages": (69_929 + 70_850) * 1024,
+    "gemv_kda_proj_1row": (197_937 + 48) * 1024,         # per launch: the weights once, the activations, the outputs
 }
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
