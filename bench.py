@@ -574,9 +574,10 @@ def bench_layer_decode(steps, warmup, stream):
         core: chain + conv window advance in one launch on the slots' states (glm53f_kda_chain_shift_batch_bf16state)
         out = kda_out x o^T     [rows][4096]
     Up to 8 rows the projections are this library's GEMV (the split one through glm53f_fwd_gemv_bf16_static, which
-    holds its scratch itself), above that the vendor GEMM, as the reference's dispatch has it (gemm.rs:228-234);
-    benchmark configuration 1's 16 slots therefore take the vendor GEMM, and 8 slots are measured beside them for
-    the GEMV path. Each both ways: launched eagerly, and as one captured graph replayed."""
+    holds its scratch itself); above that the reference's dispatch calls the vendor GEMM (gemm.rs:228-234), and this
+    library has its weight-streaming GEMM for 9 to 64 rows (glm53f_fwd_gemm_bf16_skinny). Benchmark configuration
+    1's 16 slots are measured with both, and 8 slots beside them for the GEMV path. Each both ways: launched
+    eagerly, and as one captured graph replayed."""
     from glm53f_forward import ffi as fwd
     heads, layers, slots_n, hidden = HEADS, LAYERS, 48, 4096
     width, dim = heads * DK, DK                            # 8192, 128
@@ -605,7 +606,7 @@ def bench_layer_decode(steps, warmup, stream):
     res = {"config": {"workload": "a KDA layer's decode step end to end, 34 layers in turn: kda_proj, the two gate "
                                   "projections, chain + conv window advance, o_proj; engine strides",
                       "weight_bytes_per_layer": weight_bytes}}
-    for batch in (16, 8):
+    for batch, kind, key in ((16, "skinny", "slots16"), (16, "vendor", "slots16_vendor_gemm"), (8, "gemv", "slots8")):
         normed = torch.randn(batch, hidden, device=DEV, generator=gen).to(torch.bfloat16)
         pbuf = torch.zeros(batch, pcols, dtype=torch.bfloat16, device=DEV)
         fga = torch.zeros(batch, 2 * dim, dtype=torch.bfloat16, device=DEV)
@@ -619,8 +620,8 @@ def bench_layer_decode(steps, warmup, stream):
         core_args = [(heads, batch, ptr(cu), ptr(pbuf), pcols, 3 * width, ptr(ag), 2 * width, ptr(ag, width), 2 * width,
                       ptr(convs[l]), ptr(coff), ptr(layer.conv_w), ptr(pools[l]), ptr(pools[l]), ptr(soff),
                       *layer.args(), ptr(kda_out), width, None, None, None, None, st) for l in range(layers)]
-        gemv = batch <= 8
-        if gemv:
+        gemv = kind != "vendor"
+        if kind == "gemv":
             ks = {name: fwd.glm53f_fwd_gemv_ksplit(g, nn, kk) for name, g, nn, kk in
                   (("qkvb", 1, pcols, hidden), ("fga", 1, 2 * dim, hidden), ("fgb", 2, width, dim), ("o", 1, hidden, width))}
             gv = fwd.glm53f_fwd_gemv_bf16_static
@@ -629,6 +630,14 @@ def bench_layer_decode(steps, warmup, stream):
                 (ptr(normed), hidden, 0, ptr(w_fga[l]), hidden, 0, 1, batch, 2 * dim, hidden, ks["fga"], ptr(fga), 0, 2 * dim, 0, st),
                 (ptr(fga), 2 * dim, dim, ptr(w_fgb[l]), dim, width * dim, 2, batch, width, dim, ks["fgb"], ptr(ag), 0, 2 * width, width, st),
                 (ptr(kda_out), width, 0, ptr(w_o[l]), width, 0, 1, batch, hidden, width, ks["o"], ptr(attn_out), 0, hidden, 0, st),
+            ] for l in range(layers)]
+        elif kind == "skinny":
+            gv = fwd.glm53f_fwd_gemm_bf16_skinny
+            gemv_args = [[
+                (ptr(normed), hidden, 0, ptr(w_qkvb[l]), hidden, 0, 1, batch, pcols, hidden, ptr(pbuf), 0, pcols, 0, st),
+                (ptr(normed), hidden, 0, ptr(w_fga[l]), hidden, 0, 1, batch, 2 * dim, hidden, ptr(fga), 0, 2 * dim, 0, st),
+                (ptr(fga), 2 * dim, dim, ptr(w_fgb[l]), dim, width * dim, 2, batch, width, dim, ptr(ag), 0, 2 * width, width, st),
+                (ptr(kda_out), width, 0, ptr(w_o[l]), width, 0, 1, batch, hidden, width, ptr(attn_out), 0, hidden, 0, st),
             ] for l in range(layers)]
         ag_f, ag_g = ag[:, :width], ag[:, width:]
 
@@ -659,8 +668,9 @@ def bench_layer_decode(steps, warmup, stream):
             ms_graph = timed(graph.replay, steps, warmup, stream)
         state_bytes = 2 * batch * n * 2
         per_layer = weight_bytes + state_bytes
-        key = f"slots{batch}"
-        res[key] = {"projections": "this library's GEMV (glm53f_fwd_gemv_bf16_static)" if gemv else "vendor GEMM (hipBLASLt through torch.mm)",
+        res[key] = {"projections": {"gemv": "this library's GEMV (glm53f_fwd_gemv_bf16_static)",
+                                    "skinny": "this library's GEMM for 9 to 64 rows (glm53f_fwd_gemm_bf16_skinny)",
+                                    "vendor": "vendor GEMM (hipBLASLt through torch.mm)"}[kind],
                     "eager_us_per_layer": ms_eager * 1e3 / layers, "graph_us_per_layer": ms_graph * 1e3 / layers,
                     "bytes_per_layer": per_layer, "state_bytes_per_layer": state_bytes,
                     "eager_GBps": per_layer / (ms_eager * 1e-3 / layers) / 1e9,

@@ -43,6 +43,9 @@ class Bf16Mat:
 @dataclass(frozen=True)
 class GemmPolicy:
     gemv_max_rows: int = 8
+    # rows from gemv_max_rows + 1 up to this take the library's skinny GEMM where its shape rules allow (0: never,
+    # the reference's dispatch: everything above the GEMV goes to the vendor GEMM)
+    skinny_max_rows: int = 64
 
 
 class Gemm:
@@ -70,8 +73,24 @@ class Gemm:
             return
         if rows <= self.policy.gemv_max_rows:
             self.gemv(x, ldx, x_gstride, w, rows, out, ldo, o_gstride, out_f32, stream)
+        elif rows <= self.policy.skinny_max_rows and self.skinny_takes(w, ldo, o_gstride, out_f32):
+            self.skinny(x, ldx, x_gstride, w, rows, out, ldo, o_gstride, out_f32, stream)
         else:
             self.blas(x, ldx, x_gstride, w, rows, out, ldo, o_gstride, out_f32)
+
+    @staticmethod
+    def skinny_takes(w: Bf16Mat, ldo: int, o_gstride: int, out_f32: bool) -> bool:
+        """The shapes glm53f_fwd_gemm_bf16_skinny accepts (include/glm53f_fwd_gemv.h); others go to the vendor GEMM."""
+        return w.n % 16 == 0 and w.k % 128 == 0 and (out_f32 or (ldo % 2 == 0 and o_gstride % 2 == 0))
+
+    def skinny(self, x: int, ldx: int, x_gstride: int, w: Bf16Mat, rows: int, out: int, ldo: int, o_gstride: int,
+               out_f32: bool, stream: int = 0) -> None:
+        """The weight-streaming MFMA GEMM for 9 to 64 rows (no counterpart in the reference, which calls cuBLAS
+        here: gemm.rs:228-234)."""
+        rc = ffi.glm53f_fwd_gemm_bf16_skinny(x, ldx, x_gstride, w.ptr, w.ld, w.gstride, w.groups, rows, w.n, w.k, out,
+                                             int(out_f32), ldo, o_gstride, stream)
+        if rc != 0:
+            raise GemmError("glm53f_fwd_gemm_bf16_skinny rejected its arguments" if rc == 1 else f"glm53f_fwd_gemm_bf16_skinny: hipError {rc}")
 
     def gemv(self, x: int, ldx: int, x_gstride: int, w: Bf16Mat, rows: int, out: int, ldo: int, o_gstride: int,
              out_f32: bool, stream: int = 0) -> None:

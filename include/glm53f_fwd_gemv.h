@@ -57,6 +57,22 @@ int32_t glm53f_fwd_gemv_bf16_static(const uint16_t* x, int64_t ldx, int64_t x_gs
                                     int32_t k, int32_t ksplit, void* out, int32_t out_f32, int64_t ldo,
                                     int64_t o_gstride, struct ihipStream_t* stream);
 
+/** out[g][m][o] = sum_k x[g][m][k] * w[g][o][k] for 9 to 64 rows (1 to 64 are accepted), with the weights streamed
+ *  from HBM once like the GEMV's and the arithmetic on the matrix cores (v_mfma_f32_16x16x32_bf16). It has no
+ *  counterpart in the reference's kernel ABI: above 8 rows the reference's engine calls the vendor GEMM
+ *  (crates/glm53f-forward/src/gemm.rs:228-234, `Gemm::cublas` :293-325); this is what `Gemm::bf16` can call in
+ *  its place for up to 64 rows (a decode step of 9 to 64 slots, a verify window), where the vendor's tiles leave
+ *  close to half of the weight stream's rate unused (4096 -> 24,640 with sixteen rows: 52 us there, 31 us here). Arguments as glm53f_fwd_gemv_bf16 without the split and its scratch.
+ *  n % 16 == 0, k % 128 == 0, ldx, ldw, x_gstride, w_gstride % 8 == 0, x and w 16-byte aligned, out 4-byte aligned,
+ *  ldo and o_gstride even for bf16 outputs; anything else is rejected (1) and belongs to the vendor GEMM.
+ *  Numerics: exact bf16 products, f32 accumulation over K in steps of 32 inside eighths or quarters of the K range
+ *  (or the whole of it; n and k alone decide), those added in order; bf16 outputs rounded to nearest even. Results do not depend on `rows` beyond the row's own
+ *  inputs; there is no bit-level contract with the GEMV (the reference has none between its GEMV and cuBLAS:
+ *  tests/gemv.rs holds the two together within f32 rounding, and tests/test_gpu_gemm_skinny.py does the same). */
+int32_t glm53f_fwd_gemm_bf16_skinny(const uint16_t* x, int64_t ldx, int64_t x_gstride, const uint16_t* w, int64_t ldw,
+                                    int64_t w_gstride, int32_t groups, int32_t rows, int32_t n, int32_t k, void* out,
+                                    int32_t out_f32, int64_t ldo, int64_t o_gstride, struct ihipStream_t* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -108,7 +108,8 @@ def declarations():
 
 def test_library_exports_the_declared_gemv_entry_points():
     decl = declarations()
-    assert decl == {"glm53f_fwd_gemv_bf16": 18, "glm53f_fwd_gemv_ksplit": 3, "glm53f_fwd_gemv_bf16_static": 16}
+    assert decl == {"glm53f_fwd_gemv_bf16": 18, "glm53f_fwd_gemv_ksplit": 3, "glm53f_fwd_gemv_bf16_static": 16,
+                    "glm53f_fwd_gemm_bf16_skinny": 15}
     lib = fwd.lib()
     for name, nargs in decl.items():
         assert hasattr(lib, name) and len(fwd.PROTOTYPES[name][1]) == nargs, name
