@@ -561,6 +561,51 @@ def bench_gemv(steps, warmup, stream, cpu=True):
     return res
 
 
+# ------------------------------------------------------------------------------------------------ skinny GEMM
+
+def bench_skinny(steps, warmup, stream):
+    """The same projections with 9 to 64 rows (a decode step of more than 8 slots, a verify window): this library's
+    weight-streaming GEMM (glm53f_fwd_gemm_bf16_skinny) and, beside it, the vendor GEMM that the reference's dispatch
+    takes there (crates/glm53f-forward/src/gemm.rs:228-234). The KDA layer's four projections with the engine's
+    strides; four copies of each weight in turn, so that no call finds its weight in the 256 MB Infinity Cache."""
+    from glm53f_forward import ffi as fwd
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    res = {"config": {"workload": "BF16 GEMM with 16 to 64 rows, weights [n][k] streamed once: kda_proj 4096 -> 24,640, "
+                                  "o_proj 8192 -> 4096, the gates' 4096 -> 256 and 2 x (128 -> 8192); four weight copies in turn"}}
+    copies = 4
+    for name, g, n, k, ldx, xgs, ldo, ogs, rows_list in (("kda_proj", 1, 24_640, 4096, 4096, 0, 24_640, 0, (16, 32, 64)),
+                                                         ("o_proj", 1, 4096, 8192, 8192, 0, 4096, 0, (16, 64)),
+                                                         ("fga", 1, 256, 4096, 4096, 0, 256, 0, (16,)),
+                                                         ("fgb", 2, 8192, 128, 256, 128, 16_384, 8192, (16,))):
+        w = (torch.randn(copies, g, n, k, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
+        x = torch.randn(64, ldx, device=DEV, generator=gen).to(torch.bfloat16)
+        out = torch.zeros(64, ldo, dtype=torch.bfloat16, device=DEV)
+        wbytes = g * n * k * 2
+        for rows in rows_list:
+            calls = [(ptr(x), ldx, xgs, ptr(w[c]), k, n * k, g, rows, n, k, ptr(out), 0, ldo, ogs, stream.cuda_stream)
+                     for c in range(copies)]
+            turn = [0]
+
+            def one():
+                turn[0] += 1
+                check(fwd.glm53f_fwd_gemm_bf16_skinny(*calls[turn[0] % copies]), "skinny GEMM")
+
+            ms = timed(one, steps, warmup, stream)
+            res[f"{name}_{rows}rows"] = {"us": ms * 1e3, "weight_GBps": wbytes / (ms * 1e-3) / 1e9,
+                                         "frac_of_hbm_peak": wbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+            if g == 1:
+                def vendor():
+                    turn[0] += 1
+                    torch.mm(x[:rows, :k], w[turn[0] % copies, 0].t(), out=out[:rows, :n])
+                ms = timed(vendor, steps, warmup, stream)
+                res[f"{name}_{rows}rows"]["vendor_gemm_us"] = ms * 1e3
+        del w
+    r = res["kda_proj_16rows"]
+    res["roofline"] = {"bound": "hbm", "kernel": "stream_kernel<256 k per chunk, 1 row tile, 8 weight tiles, 4 waves>",
+                       "achieved": r["weight_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": r["frac_of_hbm_peak"],
+                       "traffic": TRAFFIC_BYTES.get("skinny_kda_proj_16rows"), "algorithmic_bytes": 24_640 * 4096 * 2}
+    return res
+
 
 # ------------------------------------------------------------------------------------------------ decode layer
 
@@ -702,7 +747,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "gemv", "layer", "copy"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "verify", "mark", "gemv", "skinny", "layer", "copy"], default=None)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -758,6 +803,12 @@ def main():
         if args.only == "gemv":
             line.update({"value": gv["roofline"]["achieved"], "ms_per_step": gv["kda_proj_1row"]["us"] / 1e3,
                          "roofline": gv["roofline"], "config": gv["config"]})
+    if args.only in (None, "skinny"):
+        sk = bench_skinny(args.steps, args.warmup, stream)
+        line["skinny_gemm"] = sk
+        if args.only == "skinny":
+            line.update({"value": sk["roofline"]["achieved"], "ms_per_step": sk["kda_proj_16rows"]["us"] / 1e3,
+                         "roofline": sk["roofline"], "config": sk["config"]})
     if args.only in (None, "layer"):
         ly = bench_layer_decode(max(2, args.steps // 4), max(1, args.warmup // 2), stream)
         line["layer_decode"] = ly

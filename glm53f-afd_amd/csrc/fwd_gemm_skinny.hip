@@ -211,7 +211,7 @@ int32_t launch_tiles(const Args& a) {
 // The K split depends on n and k alone, so a row's bits do not change with the number of rows beside it: eight waves
 // where the grid is at most one workgroup per CU even at one tile each (more loads in flight per CU), four otherwise,
 // one where the K range is too short to split into chunks. The chunk is 256 k where sixteen rows leave the
-// registers for it and the wave's range is a multiple of it.
+// registers for it and the wave's range is a multiple of it (32 rows still do where the K range is split in four).
 template <int NT, int TMAX>
 int32_t launch_split(const Args& a) {
     const long long tiles = (long long)(a.n / 16) * a.groups;
@@ -220,7 +220,7 @@ int32_t launch_split(const Args& a) {
         return launch<128, NT, 1, 8>(a);
     }
     if (a.k % (4 * 128) == 0) {
-        if constexpr (NT == 1) if (a.k % (4 * 256) == 0) return launch_tiles<256, 1, 4, TMAX>(a);
+        if constexpr (NT <= 2) if (a.k % (4 * 256) == 0) return launch_tiles<256, NT, 4, TMAX>(a);
         return launch_tiles<128, NT, 4, TMAX>(a);
     }
     return launch_tiles<128, NT, 1, TMAX>(a);
@@ -247,7 +247,7 @@ extern "C" int32_t glm53f_fwd_gemm_bf16_skinny(const uint16_t* x, int64_t ldx, i
     switch ((rows + 15) / 16) {                   // the accumulators (4 T NT registers) bound T
         case 1: return launch_split<1, 8>(a);
         case 2: return launch_split<2, 4>(a);
-        case 3: return launch_split<3, 2>(a);
-        default: return launch_split<4, 2>(a);
+        default: return launch_split<4, 4>(a);    // 33 to 48 rows too: a third tile's seven items per chunk need more
+                                                  // registers than a fourth tile of repeated rows costs
     }
 }
