@@ -35,11 +35,12 @@ from glm53f_kda import DK, DV, HEADS, LAYERS, WINDOW, channels, ffi, state_len
 # offline; the summaries are kept in profiles/.
 TRAFFIC_BYTES = {
     "decode_chain": (36_798 + 33_024) * 1024,            # per plain chain launch, 16 slots x 1 row
-    "verify_chain": (167_883 + 1_585_706) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
+    "verify_chain": (167_884 + 1_585_717) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
     # two passes of 1024 rows (intra read + written, inter read + written) and one norm launch
-    "prefill_2048_rows": (2 * (74_012 + 141_316 + 144_138 + 20_482) + 65_755 + 32_912) * 1024,
-    "mark_state_pages": (69_929 + 70_850) * 1024,
-    "gemv_kda_proj_1row": (197_937 + 48) * 1024,         # per launch: the weights once, the activations, the outputs
+    "prefill_2048_rows": (2 * (74_010 + 141_326 + 144_138 + 20_482) + 65_755 + 32_912) * 1024,
+    "mark_state_pages": (69_934 + 70_858) * 1024,
+    "gemv_kda_proj_1row": (197_928 + 48) * 1024,         # per launch: the weights once, the activations, the outputs
+    "skinny_kda_proj_16rows": (198_457 + 770) * 1024,    # per launch: the weights once, sixteen rows' activations per workgroup (L2), the outputs
 }
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
@@ -621,8 +622,10 @@ def bench_layer_decode(steps, warmup, stream):
     Up to 8 rows the projections are this library's GEMV (the split one through glm53f_fwd_gemv_bf16_static, which
     holds its scratch itself); above that the reference's dispatch calls the vendor GEMM (gemm.rs:228-234), and this
     library has its weight-streaming GEMM for 9 to 64 rows (glm53f_fwd_gemm_bf16_skinny). Benchmark configuration
-    1's 16 slots are measured with both, and 8 slots beside them for the GEMV path. Each both ways: launched
-    eagerly, and as one captured graph replayed."""
+    1's 16 slots are measured with both, and 8 slots beside them for the GEMV path (and with the GEMM for 9 to 64
+    rows, which accepts fewer: the reference's bit-level contract with its host model is then given up, a row's
+    independence of the rows beside it is not). Each both ways: launched eagerly, and as one captured graph
+    replayed."""
     from glm53f_forward import ffi as fwd
     heads, layers, slots_n, hidden = HEADS, LAYERS, 48, 4096
     width, dim = heads * DK, DK                            # 8192, 128
@@ -651,7 +654,8 @@ def bench_layer_decode(steps, warmup, stream):
     res = {"config": {"workload": "a KDA layer's decode step end to end, 34 layers in turn: kda_proj, the two gate "
                                   "projections, chain + conv window advance, o_proj; engine strides",
                       "weight_bytes_per_layer": weight_bytes}}
-    for batch, kind, key in ((16, "skinny", "slots16"), (16, "vendor", "slots16_vendor_gemm"), (8, "gemv", "slots8")):
+    for batch, kind, key in ((16, "skinny", "slots16"), (16, "vendor", "slots16_vendor_gemm"), (8, "gemv", "slots8"),
+                             (8, "skinny", "slots8_skinny_gemm")):
         normed = torch.randn(batch, hidden, device=DEV, generator=gen).to(torch.bfloat16)
         pbuf = torch.zeros(batch, pcols, dtype=torch.bfloat16, device=DEV)
         fga = torch.zeros(batch, 2 * dim, dtype=torch.bfloat16, device=DEV)
