@@ -654,21 +654,35 @@ def bench_layer_decode(steps, warmup, stream):
     res = {"config": {"workload": "a KDA layer's decode step end to end, 34 layers in turn: kda_proj, the two gate "
                                   "projections, chain + conv window advance, o_proj; engine strides",
                       "weight_bytes_per_layer": weight_bytes}}
-    for batch, kind, key in ((16, "skinny", "slots16"), (16, "vendor", "slots16_vendor_gemm"), (8, "gemv", "slots8"),
-                             (8, "skinny", "slots8_skinny_gemm")):
+    ck = None
+    # (slots, rows per slot, who runs the projections, key): one row per slot is a decode step; four rows per slot a
+    # verify window (the core is then glm53f_kda_verify_batch_bf16state with a checkpoint after every row, which
+    # leaves the slots' states and windows as they are: the commit is the select of the verify leg)
+    for slots, per, kind, key in ((16, 1, "skinny", "slots16"), (16, 1, "vendor", "slots16_vendor_gemm"), (8, 1, "gemv", "slots8"),
+                                  (8, 1, "skinny", "slots8_skinny_gemm"), (16, 4, "skinny", "verify_16slots_x4"),
+                                  (16, 4, "vendor", "verify_16slots_x4_vendor_gemm")):
+        batch = slots * per
         normed = torch.randn(batch, hidden, device=DEV, generator=gen).to(torch.bfloat16)
         pbuf = torch.zeros(batch, pcols, dtype=torch.bfloat16, device=DEV)
         fga = torch.zeros(batch, 2 * dim, dtype=torch.bfloat16, device=DEV)
         ag = torch.zeros(batch, 2 * width, dtype=torch.bfloat16, device=DEV)
         kda_out = torch.zeros(batch, width, dtype=torch.bfloat16, device=DEV)
         attn_out = torch.zeros(batch, hidden, dtype=torch.bfloat16, device=DEV)
-        perm = torch.randperm(slots_n, generator=torch.Generator().manual_seed(12))[:batch]
-        cu = torch.arange(batch + 1, dtype=torch.int32, device=DEV)
+        perm = torch.randperm(slots_n, generator=torch.Generator().manual_seed(12))[:slots]
+        cu = (torch.arange(slots + 1, dtype=torch.int32) * per).to(DEV)
         soff, coff = (perm.to(torch.int64) * n).to(DEV), (perm.to(torch.int64) * cw).to(DEV)
-        core = ffi.glm53f_kda_chain_shift_batch_bf16state
-        core_args = [(heads, batch, ptr(cu), ptr(pbuf), pcols, 3 * width, ptr(ag), 2 * width, ptr(ag, width), 2 * width,
-                      ptr(convs[l]), ptr(coff), ptr(layer.conv_w), ptr(pools[l]), ptr(pools[l]), ptr(soff),
-                      *layer.args(), ptr(kda_out), width, None, None, None, None, st) for l in range(layers)]
+        if per == 1:
+            core = ffi.glm53f_kda_chain_shift_batch_bf16state
+            core_args = [(heads, slots, ptr(cu), ptr(pbuf), pcols, 3 * width, ptr(ag), 2 * width, ptr(ag, width), 2 * width,
+                          ptr(convs[l]), ptr(coff), ptr(layer.conv_w), ptr(pools[l]), ptr(pools[l]), ptr(soff),
+                          *layer.args(), ptr(kda_out), width, None, None, None, None, st) for l in range(layers)]
+        else:
+            if ck is None:
+                ck = torch.empty(layers, batch * n, dtype=torch.bfloat16, device=DEV)   # a checkpoint per row and layer
+            core = ffi.glm53f_kda_verify_batch_bf16state
+            core_args = [(heads, slots, ptr(cu), ptr(pbuf), pcols, 3 * width, ptr(ag), 2 * width, ptr(ag, width), 2 * width,
+                          ptr(convs[l]), ptr(coff), ptr(layer.conv_w), ptr(pools[l]), ptr(soff),
+                          *layer.args(), ptr(kda_out), width, ptr(ck[l]), None, None, None, None, st) for l in range(layers)]
         gemv = kind != "vendor"
         if kind == "gemv":
             ks = {name: fwd.glm53f_fwd_gemv_ksplit(g, nn, kk) for name, g, nn, kk in
@@ -715,7 +729,7 @@ def bench_layer_decode(steps, warmup, stream):
             with torch.cuda.graph(graph, stream=stream):
                 step()
             ms_graph = timed(graph.replay, steps, warmup, stream)
-        state_bytes = 2 * batch * n * 2
+        state_bytes = (2 * slots if per == 1 else slots + batch) * n * 2     # read + written | read + checkpoints
         per_layer = weight_bytes + state_bytes
         res[key] = {"projections": {"gemv": "this library's GEMV (glm53f_fwd_gemv_bf16_static)",
                                     "skinny": "this library's GEMM for 9 to 64 rows (glm53f_fwd_gemm_bf16_skinny)",
@@ -727,7 +741,8 @@ def bench_layer_decode(steps, warmup, stream):
         best = min(ms_eager, ms_graph)
         res[key]["roofline"] = {"bound": "hbm", "achieved": per_layer / (best * 1e-3 / layers) / 1e9, "peak": HBM_PEAK_GBPS,
                                 "unit": "GB/s", "frac": per_layer / (best * 1e-3 / layers) / 1e9 / HBM_PEAK_GBPS,
-                                "traffic": None, "what": "weights of the four projections + state read and written, "
+                                "traffic": None, "what": "weights of the four projections + state read and written (a verify "
+                                                         "window: read, and a checkpoint written per row), "
                                                          "over the faster of the eager and the graph time"}
         del graph
     return res
