@@ -210,8 +210,11 @@ int32_t launch_tiles(const Args& a) {
 
 // The K split depends on n and k alone, so a row's bits do not change with the number of rows beside it: eight waves
 // where the grid is at most one workgroup per CU even at one tile each (more loads in flight per CU), four otherwise,
-// one where the K range is too short to split into chunks. The chunk is 256 k where sixteen rows leave the
-// registers for it and the wave's range is a multiple of it (32 rows still do where the K range is split in four).
+// one where the K range is too short to split into chunks. The chunk is 256 k where the wave's range is a multiple
+// of it and, with eight waves, where sixteen rows leave the registers for it; with four waves the workgroup may
+// run alone on its CU (eight weight tiles x four row tiles: 426 registers, the accumulators in the AGPRs), which
+// pays because the activations' L2 traffic falls with the tiles per workgroup: 4096 -> 24,640 with 64 rows
+// 38 us at eight tiles against 45 at four.
 template <int NT, int TMAX>
 int32_t launch_split(const Args& a) {
     const long long tiles = (long long)(a.n / 16) * a.groups;
@@ -220,7 +223,7 @@ int32_t launch_split(const Args& a) {
         return launch<128, NT, 1, 8>(a);
     }
     if (a.k % (4 * 128) == 0) {
-        if constexpr (NT <= 2) if (a.k % (4 * 256) == 0) return launch_tiles<256, NT, 4, TMAX>(a);
+        if (a.k % (4 * 256) == 0) return launch_tiles<256, NT, 4, 8>(a);
         return launch_tiles<128, NT, 4, TMAX>(a);
     }
     return launch_tiles<128, NT, 1, TMAX>(a);
@@ -244,7 +247,7 @@ extern "C" int32_t glm53f_fwd_gemm_bf16_skinny(const uint16_t* x, int64_t ldx, i
     if (!out_f32 && ((reinterpret_cast<uintptr_t>(out) & 3u) || ldo % 2 || o_gstride % 2)) return kInvalid;
     if (out_f32 && (reinterpret_cast<uintptr_t>(out) & 3u)) return kInvalid;
     const Args a{x, ldx, x_gstride, w, ldw, w_gstride, groups, rows, n, k, out, out_f32, ldo, o_gstride, stream};
-    switch ((rows + 15) / 16) {                   // the accumulators (4 T NT registers) bound T
+    switch ((rows + 15) / 16) {                   // (the last argument bounds T where the chunk is 128 k)
         case 1: return launch_split<1, 8>(a);
         case 2: return launch_split<2, 4>(a);
         default: return launch_split<4, 4>(a);    // 33 to 48 rows too: a third tile's seven items per chunk need more
