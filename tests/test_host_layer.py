@@ -1,6 +1,7 @@
 """The C++ host layer (glm53f-afd_amd/host: the counterpart of the reference's kernel.rs / device.rs and of the BF16
-half of the forward crate's gemm.rs / cublas.rs) through its test programs, tests/host/host_tests.cc and
-gemm_tests.cc: argument checks and shape rules without a GPU, launches against the oracle with one."""
+half of the forward crate's gemm.rs / cublas.rs and of the KDA layer's call site in forward.rs) through its test
+programs, tests/host/host_tests.cc, gemm_tests.cc and kda_layer_tests.cc: argument checks and shape rules without a
+GPU, launches against the oracle and against each other with one."""
 import os
 import subprocess
 
@@ -10,6 +11,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HOST = os.path.join(ROOT, "tests", "host")
 EXE = os.path.join(HOST, "host_tests")
 GEMM_EXE = os.path.join(HOST, "gemm_tests")
+LAYER_EXE = os.path.join(HOST, "kda_layer_tests")
 
 
 def _exe(path=EXE):
@@ -38,5 +40,17 @@ def test_gemm_engine_policy_and_shape_rules_without_a_gpu():
 @pytest.mark.gpu
 def test_gemm_engine_dispatch_matches_exact_arithmetic():
     r = subprocess.run([_exe(GEMM_EXE), "--gpu"], capture_output=True, text=True, timeout=300)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout + r.stderr
+
+
+def test_kda_call_site_shapes_without_a_gpu():
+    r = subprocess.run([_exe(LAYER_EXE), "--cpu"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+
+
+@pytest.mark.gpu
+def test_kda_call_site_verify_commit_and_prefill():
+    r = subprocess.run([_exe(LAYER_EXE), "--gpu"], capture_output=True, text=True, timeout=300)
     print(r.stdout)
     assert r.returncode == 0, r.stdout + r.stderr
