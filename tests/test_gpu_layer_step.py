@@ -37,27 +37,36 @@ class Layer:
         self.state = rnd(POOL * N, scale=0.05)
         self.conv = rnd(POOL * CW, scale=1.0)
 
-    def step(self, gemm, x, meta, state, conv, ckpt=None):
-        """x [rows][HIDDEN] bf16 -> attention output [rows][HIDDEN]; ckpt None: a decode round in place (chain + conv
-        window advance), else a verify window that leaves state and conv alone and writes a checkpoint per row."""
-        rows = x.shape[0]
+    @staticmethod
+    def buffers(rows):
         z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
-        p, fga, ag, kda_out, out = z(rows, P_COLS), z(rows, 2 * DK), z(rows, 2 * WIDTH), z(rows, WIDTH), z(rows, HIDDEN)
-        gemm.bf16(hs.ptr(x), HIDDEN, 0, Bf16Mat.of(self.qkvb), rows, hs.ptr(p), P_COLS, 0, False)
-        gemm.bf16(hs.ptr(x), HIDDEN, 0, Bf16Mat.of(self.fga), rows, hs.ptr(fga), 2 * DK, 0, False)
-        gemm.bf16(hs.ptr(fga), 2 * DK, DK, Bf16Mat.of(self.fgb), rows, hs.ptr(ag), 2 * WIDTH, WIDTH, False)
+        return dict(p=z(rows, P_COLS), fga=z(rows, 2 * DK), ag=z(rows, 2 * WIDTH), kda_out=z(rows, WIDTH), out=z(rows, HIDDEN))
+
+    def launch(self, gemm, x, meta, state, conv, b, ckpt=None, stream=None):
+        """The step's five launches on `stream` into the row buffers b (no allocation, no synchronisation)."""
+        rows = x.shape[0]
+        p, fga, ag, kda_out, out = b["p"], b["fga"], b["ag"], b["kda_out"], b["out"]
+        gemm.bf16(hs.ptr(x), HIDDEN, 0, Bf16Mat.of(self.qkvb), rows, hs.ptr(p), P_COLS, 0, False, stream)
+        gemm.bf16(hs.ptr(x), HIDDEN, 0, Bf16Mat.of(self.fga), rows, hs.ptr(fga), 2 * DK, 0, False, stream)
+        gemm.bf16(hs.ptr(fga), 2 * DK, DK, Bf16Mat.of(self.fgb), rows, hs.ptr(ag), 2 * WIDTH, WIDTH, False, stream)
         w = self.kda
         head = [H, meta.batch, hs.ptr(meta.cu_rows), hs.ptr(p), P_COLS, C, hs.ptr(ag), 2 * WIDTH, hs.ptr(ag, WIDTH), 2 * WIDTH,
                 hs.ptr(conv), hs.ptr(meta.conv_off), hs.ptr(w.conv_w), hs.ptr(state)]
         if ckpt is None:
             hs.check(ffi.glm53f_kda_chain_shift_batch_bf16state(*head, hs.ptr(state), hs.ptr(meta.state_off), *w.args(),
-                                                                hs.ptr(kda_out), WIDTH, None, None, None, None, None), "decode")
+                                                                hs.ptr(kda_out), WIDTH, None, None, None, None, stream), "decode")
         else:
             hs.check(ffi.glm53f_kda_verify_batch_bf16state(*head, hs.ptr(meta.state_off), *w.args(), hs.ptr(kda_out), WIDTH,
-                                                           hs.ptr(ckpt), None, None, None, None, None), "verify")
-        gemm.bf16(hs.ptr(kda_out), WIDTH, 0, Bf16Mat.of(self.o), rows, hs.ptr(out), HIDDEN, 0, False)
+                                                           hs.ptr(ckpt), None, None, None, None, stream), "verify")
+        gemm.bf16(hs.ptr(kda_out), WIDTH, 0, Bf16Mat.of(self.o), rows, hs.ptr(out), HIDDEN, 0, False, stream)
+
+    def step(self, gemm, x, meta, state, conv, ckpt=None):
+        """x [rows][HIDDEN] bf16 -> attention output [rows][HIDDEN]; ckpt None: a decode round in place (chain + conv
+        window advance), else a verify window that leaves state and conv alone and writes a checkpoint per row."""
+        b = self.buffers(x.shape[0])
+        self.launch(gemm, x, meta, state, conv, b, ckpt)
         hs.sync()
-        return out, p
+        return b["out"], b["p"]
 
 
 @pytest.mark.parametrize("slots_n,drafts", [(16, 4), (5, 3), (3, 16)])
@@ -111,3 +120,36 @@ def test_the_default_dispatch_agrees_with_the_reference_dispatch_within_bf16_rou
     worst = float((outs[0] - outs[1]).abs().max())
     print(f"layer output, skinny against vendor GEMM: max |diff| {worst:.3e} at max |out| {scale:.3e}")
     assert worst <= 2.0 ** -5 * scale
+
+
+@pytest.mark.parametrize("rows", [8, 16])
+def test_a_captured_layer_step_replays_like_eager_steps(rows):
+    """The step's five launches recorded once (8 rows: the GEMV, whose split projection uses the engine's counters;
+    16 rows: the GEMM for 9 to 64 rows) and replayed: nothing on the path allocates or clears with a memset. Every
+    replay advances the slots' states and windows, and is held to the same step made eagerly, bit for bit, with eager
+    work and synchronisations between the replays."""
+    layer_g, layer_e = Layer(91), Layer(91)
+    assert torch.equal(layer_g.state, layer_e.state)
+    gemm = Gemm()
+    g = torch.Generator(device=DEV).manual_seed(9)
+    slots = list(range(2, 2 + rows))
+    x = torch.randn(rows, HIDDEN, device=DEV, generator=g).to(torch.bfloat16)
+    one = hs.BatchMeta([1] * rows, [s * CW for s in slots], [s * N for s in slots])
+    bg, be = Layer.buffers(rows), Layer.buffers(rows)
+    stream = torch.cuda.Stream()                       # default priority; the legacy default stream cannot be captured
+    hs.sync()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            layer_g.launch(gemm, x, one, layer_g.state, layer_g.conv, bg, stream=stream.cuda_stream)
+        for replay in range(1, 4):
+            graph.replay()
+            stream.synchronize()
+            layer_e.launch(gemm, x, one, layer_e.state, layer_e.conv, be, stream=stream.cuda_stream)
+            junk = torch.randn(1 << 16, device=DEV).sum().item()
+            hs.sync()
+            assert junk == junk
+            assert torch.equal(bg["out"], be["out"]), f"attention outputs of replay {replay}"
+            assert torch.equal(layer_g.state, layer_e.state), f"states after replay {replay}"
+            assert torch.equal(layer_g.conv, layer_e.conv), f"conv windows after replay {replay}"
+    assert not torch.equal(layer_g.state, Layer(91).state)
