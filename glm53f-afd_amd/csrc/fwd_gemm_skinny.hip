@@ -72,6 +72,8 @@ __global__ void __launch_bounds__(64 * KS) stream_kernel(const uint16_t* __restr
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int g = blockIdx.z, tiles = n / 16, tile0 = blockIdx.x * T;
+    const int row0 = blockIdx.y * (16 * NT);      // gridDim.y > 1: the rows in groups of 16 NT, a workgroup each
+    rows = min(rows - row0, 16 * NT);
     const int kc = k / KS, lo = wave * kc, chunks = kc / CK;
     const int lrow = lane / S::LANES, lcol = 8 * (lane % S::LANES);
     unsigned char* stage = lds + wave * S::BYTES;
@@ -80,7 +82,7 @@ __global__ void __launch_bounds__(64 * KS) stream_kernel(const uint16_t* __restr
 
     // items 0 .. NT - 1 of a chunk: the activations' tiles (a row past the end repeats the last one: its column
     // is not stored); item NT + i: weight tile i of this workgroup (a tile past the last repeats it, not stored)
-    const uint16_t* xsrc = x + g * x_gs + lo + lcol;
+    const uint16_t* xsrc = x + g * x_gs + (long long)row0 * ldx + lo + lcol;
     const uint16_t* wsrc = w + g * w_gs + (long long)lrow * ldw + lo + lcol;
     auto request = [&](u32x4 (&set)[N8], int item, int c) {
         if (item < NT) {
@@ -172,10 +174,10 @@ __global__ void __launch_bounds__(64 * KS) stream_kernel(const uint16_t* __restr
         const int row = 16 * nt + (l & 15), o = 16 * (tile0 + i) + 4 * (l >> 4);
         if (row >= rows || tile0 + i >= tiles) continue;
         if (out_f32) {
-            float* dst = static_cast<float*>(out) + g * o_gs + (long long)row * ldo + o;
+            float* dst = static_cast<float*>(out) + g * o_gs + (long long)(row0 + row) * ldo + o;
             dst[0] = s[0]; dst[1] = s[1]; dst[2] = s[2]; dst[3] = s[3];
         } else {
-            uint32_t* dst = reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(out) + g * o_gs + (long long)row * ldo + o);
+            uint32_t* dst = reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(out) + g * o_gs + (long long)(row0 + row) * ldo + o);
             dst[0] = f2bf2(s[0], s[1]);
             dst[1] = f2bf2(s[2], s[3]);
         }
@@ -192,7 +194,7 @@ struct Args {
 
 template <int CK, int NT, int T, int KS>
 int32_t launch(const Args& a) {
-    const dim3 grid((unsigned)((a.n / 16 + T - 1) / T), 1, (unsigned)a.groups);
+    const dim3 grid((unsigned)((a.n / 16 + T - 1) / T), (unsigned)((a.rows + 16 * NT - 1) / (16 * NT)), (unsigned)a.groups);
     stream_kernel<CK, NT, T, KS><<<grid, 64 * KS, 0, a.stream>>>(a.x, a.ldx, a.x_gs, a.w, a.ldw, a.w_gs, a.rows, a.n, a.k,
                                                                  a.out, a.out_f32, a.ldo, a.o_gs);
     return (int32_t)hipGetLastError();
@@ -219,7 +221,10 @@ template <int NT, int TMAX>
 int32_t launch_split(const Args& a) {
     const long long tiles = (long long)(a.n / 16) * a.groups;
     if (tiles <= kCus && a.k % (8 * 128) == 0) {
-        if constexpr (NT == 1) if (a.k % (8 * 256) == 0) return launch<256, 1, 1, 8>(a);
+        // A weight so small that a workgroup per tile and per sixteen rows still leaves CUs free (the gates' first
+        // projection: 16 tiles) is bound by a wave's chain of items, not by bytes: the row tiles go to workgroups of
+        // their own, which re-read the weight from the L2 (4096 -> 256 with 64 rows: 11 -> 6.5 us).
+        if (a.k % (8 * 256) == 0 && (NT == 1 || tiles * NT <= kCus)) return launch<256, 1, 1, 8>(a);
         return launch<128, NT, 1, 8>(a);
     }
     if (a.k % (4 * 128) == 0) {
