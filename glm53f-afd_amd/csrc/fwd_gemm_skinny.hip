@@ -223,7 +223,7 @@ int32_t launch_split(const Args& a) {
     if (tiles <= kCus && a.k % (8 * 128) == 0) {
         // A weight so small that a workgroup per tile and per sixteen rows still leaves CUs free (the gates' first
         // projection: 16 tiles) is bound by a wave's chain of items, not by bytes: the row tiles go to workgroups of
-        // their own, which re-read the weight from the L2 (4096 -> 256 with 64 rows: 11 -> 6.5 us).
+        // their own, which re-read the weight from the L2 (4096 -> 256 with 64 rows: 11 -> 6 us).
         if (a.k % (8 * 256) == 0 && (NT == 1 || tiles * NT <= kCus)) return launch<256, 1, 1, 8>(a);
         return launch<128, NT, 1, 8>(a);
     }
