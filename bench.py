@@ -572,13 +572,21 @@ def bench_skinny(steps, warmup, stream):
     from glm53f_forward import ffi as fwd
     gen = torch.Generator(device=DEV).manual_seed(9)
     res = {"config": {"workload": "BF16 GEMM with 16 to 64 rows, weights [n][k] streamed once: kda_proj 4096 -> 24,640, "
-                                  "o_proj 8192 -> 4096, the gates' 4096 -> 256 and 2 x (128 -> 8192); four weight copies in turn"}}
-    copies = 4
+                                  "o_proj 8192 -> 4096, the gates' 4096 -> 256 and 2 x (128 -> 8192), the LM head "
+                                  "4096 -> 151,936; four weight copies in turn (two of the LM head)"}}
     for name, g, n, k, ldx, xgs, ldo, ogs, rows_list in (("kda_proj", 1, 24_640, 4096, 4096, 0, 24_640, 0, (16, 32, 64)),
                                                          ("o_proj", 1, 4096, 8192, 8192, 0, 4096, 0, (16, 64)),
                                                          ("fga", 1, 256, 4096, 4096, 0, 256, 0, (16,)),
-                                                         ("fgb", 2, 8192, 128, 256, 128, 16_384, 8192, (16,))):
-        w = (torch.randn(copies, g, n, k, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
+                                                         ("fgb", 2, 8192, 128, 256, 128, 16_384, 8192, (16,)),
+                                                         # the LM head, which the reference's engine sends through the
+                                                         # same BF16 dispatch (gemm.rs:3): 1.24 GB of weights
+                                                         ("lm_head", 1, 151_936, 4096, 4096, 0, 151_936, 0, (16,))):
+        copies = 4 if n * k < (1 << 28) else 2
+        w = torch.empty(copies, g, n, k, dtype=torch.bfloat16, device=DEV)
+        flat = w.view(-1)
+        for i in range(0, flat.numel(), 1 << 26):               # in slices: the f32 temporaries stay small
+            j = min(flat.numel(), i + (1 << 26))
+            flat[i:j] = (torch.randn(j - i, device=DEV, generator=gen) * 0.02).to(torch.bfloat16)
         x = torch.randn(64, ldx, device=DEV, generator=gen).to(torch.bfloat16)
         out = torch.zeros(64, ldo, dtype=torch.bfloat16, device=DEV)
         wbytes = g * n * k * 2
