@@ -35,12 +35,12 @@ from glm53f_kda import DK, DV, HEADS, LAYERS, WINDOW, channels, ffi, state_len
 # offline; the summaries are kept in profiles/.
 TRAFFIC_BYTES = {
     "decode_chain": (36_798 + 33_024) * 1024,            # per plain chain launch, 16 slots x 1 row
-    "verify_chain": (167_883 + 1_585_742) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
+    "verify_chain": (167_884 + 1_585_673) * 1024,        # per chain launch, 48 slots x 16 rows with checkpoints
     # two passes of 1024 rows (intra read + written, inter read + written) and one norm launch
-    "prefill_2048_rows": (2 * (74_008 + 141_314 + 144_138 + 20_482) + 65_755 + 32_912) * 1024,
-    "mark_state_pages": (69_931 + 70_855) * 1024,
-    "gemv_kda_proj_1row": (197_931 + 48) * 1024,         # per launch: the weights once, the activations, the outputs
-    "skinny_kda_proj_16rows": (198_452 + 770) * 1024,    # per launch: the weights once, sixteen rows' activations per workgroup (L2), the outputs
+    "prefill_2048_rows": (2 * (74_010 + 141_329 + 144_138 + 20_482) + 65_755 + 32_912) * 1024,
+    "mark_state_pages": (69_928 + 70_854) * 1024,
+    "gemv_kda_proj_1row": (197_941 + 48) * 1024,         # per launch: the weights once, the activations, the outputs
+    "skinny_kda_proj_16rows": (198_481 + 770) * 1024,    # per launch: the weights once, sixteen rows' activations per workgroup (L2), the outputs
 }
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
